@@ -1,8 +1,8 @@
 // K2, prefill regime, one wave per SIMD: Y[M, N] = epilogue(X[M, K] . W[N, K]^T).
 //
-// The 256 x 256-tile schedule of hipBLASLt's gfx950 bf16 kernels
-// (Cijk_..._MT256x256x64_MI16x16x1_..._DTLA1_DTLB1_PGR2_PLR1_..._WG32_8_1: its K loop read from
-// the disassembly of the installed library), rebuilt in HIP for our K-contiguous operands and
+// A 256 x 256-tile, one-wave-per-SIMD schedule (MT256x256x64, 16x16 MFMA, direct-to-LDS loads of
+// both operands, two-deep global prefetch, one-deep local prefetch) written in HIP for our
+// K-contiguous operands and
 // extended with the fused serving epilogues of gemm.hip and with 192 / 128-row tiles:
 //   * 256 threads = 4 waves, ONE per SIMD, as 2 (M) x 2 (N); each wave owns (BM / 2) x 128 outputs =
 //     MB x 8 v_mfma_f32_16x16x32_bf16 accumulators (MB = BM / 32: 8 / 6 / 4) pinned to AGPRs by
