@@ -1066,12 +1066,221 @@ struct XgmiAr {
   }
 };
 
-}  // namespace
+// ---------------------------------------------------------------------------------------------
+// f32 residual stream, sigmoid attention, state-space mixer (bf16 or f32 activations)
+int esz_of(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat, name, " must be bfloat16 or float32");
+  return (int)t.element_size();
+}
+void same_type(const at::Tensor& a, const at::Tensor& b, const char* name) {
+  TORCH_CHECK(a.scalar_type() == b.scalar_type(), name, ": dtype differs from the activations'");
+}
+const float* fpo(const c10::optional<at::Tensor>& t, int64_t n, const char* name) {
+  if (!t) return nullptr;
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat && t->is_contiguous() && t->numel() == n, name, " must be f32 [", n, "]");
+  return t->data_ptr<float>();
+}
+const float* fp(const at::Tensor& t, int64_t n, const char* name) { return fpo(c10::optional<at::Tensor>(t), n, name); }
 
+std::vector<at::Tensor> embed_pos(const at::Tensor& ids, const at::Tensor& positions, const at::Tensor& tok,
+                                  const at::Tensor& pos, bool keep_copy) {
+  CHECK_CUDA(ids); CHECK_I32(ids); CHECK_I32(positions); CHECK_CONTIG(ids); CHECK_CONTIG(positions);
+  const int esz = esz_of(tok, "tok");
+  same_type(tok, pos, "pos");
+  TORCH_CHECK(tok.dim() == 2 && pos.dim() == 2 && tok.is_contiguous() && pos.is_contiguous() && tok.size(1) == pos.size(1), "tables");
+  const long T = ids.numel();
+  TORCH_CHECK(positions.numel() == T, "positions");
+  const int W = tok.size(1);
+  at::Tensor x = at::empty({T, W}, tok.options().dtype(at::kFloat));
+  at::Tensor copy = keep_copy ? at::empty({T, W}, x.options()) : at::Tensor();
+  CHECK_RC(lk_embed_pos(ip(ids), ip(positions), tok.data_ptr(), tok.size(0), pos.data_ptr(), pos.size(0), T, W,
+                        x.data_ptr<float>(), keep_copy ? copy.data_ptr<float>() : nullptr, esz, cur_stream()), "embed_pos");
+  return keep_copy ? std::vector<at::Tensor>{x, copy} : std::vector<at::Tensor>{x};
+}
+
+at::Tensor stream_rmsnorm(at::Tensor& x, const c10::optional<at::Tensor>& a, const c10::optional<at::Tensor>& b,
+                          const c10::optional<at::Tensor>& e, double mult, const c10::optional<at::Tensor>& w,
+                          double woff, double eps, const c10::optional<at::Tensor>& idx, at::ScalarType out_dtype) {
+  CHECK_CUDA(x); CHECK_F32(x); CHECK_CONTIG(x);
+  TORCH_CHECK(x.dim() == 2, "x must be [T, W]");
+  const long T = x.size(0);
+  const int W = x.size(1);
+  at::Tensor out = at::empty({idx ? idx->numel() : T, W}, x.options().dtype(out_dtype));
+  const int esz = esz_of(out, "out");
+  long as = 0, bs = 0;
+  if (a) { CHECK_CUDA(*a); same_type(*a, out, "a"); CHECK_LASTDIM(*a); TORCH_CHECK(a->dim() == 2 && a->size(0) == T && a->size(1) == W, "a shape"); as = a->stride(0); }
+  if (b) { CHECK_CUDA(*b); same_type(*b, out, "b"); CHECK_LASTDIM(*b); TORCH_CHECK(b->dim() == 2 && b->size(0) == T && b->size(1) == W, "b shape"); bs = b->stride(0); }
+  if (e) { CHECK_CUDA(*e); CHECK_F32(*e); CHECK_CONTIG(*e); TORCH_CHECK(e->sizes() == x.sizes(), "e shape"); }
+  if (idx) { CHECK_CUDA(*idx); TORCH_CHECK(idx->scalar_type() == at::kLong && idx->is_contiguous(), "idx must be int64"); }
+  CHECK_RC(lk_stream_rmsnorm(x.data_ptr<float>(), a ? a->data_ptr() : nullptr, as, b ? b->data_ptr() : nullptr, bs,
+                             e ? e->data_ptr<float>() : nullptr, (float)mult, fpo(w, W, "w"), (float)woff, (float)eps,
+                             idx ? idx->data_ptr<int64_t>() : nullptr, out.size(0), out.data_ptr(), out.stride(0), W, esz,
+                             cur_stream()), "stream_rmsnorm");
+  return out;
+}
+
+at::Tensor softcap(const at::Tensor& z, double cap) {
+  CHECK_CUDA(z); CHECK_LASTDIM(z);
+  TORCH_CHECK(z.dim() == 2, "logits must be [R, V]");
+  const int esz = esz_of(z, "logits");
+  at::Tensor out = at::empty({z.size(0), z.size(1)}, z.options().dtype(at::kFloat));
+  CHECK_RC(lk_softcap(z.data_ptr(), z.stride(0), (float)cap, out.data_ptr<float>(), out.stride(0), z.size(0), z.size(1), esz,
+                      cur_stream()), "softcap");
+  return out;
+}
+
+at::Tensor silu_mul_f32(const at::Tensor& x) {
+  CHECK_CUDA(x); CHECK_F32(x); CHECK_LASTDIM(x);
+  TORCH_CHECK(x.dim() == 2 && x.size(1) % 2 == 0, "x must be [T, 2 I]");
+  const int I = x.size(1) / 2;
+  at::Tensor out = at::empty({x.size(0), I}, x.options());
+  CHECK_RC(lk_silu_mul_f32(x.data_ptr<float>(), x.stride(0), out.data_ptr<float>(), out.stride(0), x.size(0), I, cur_stream()),
+           "silu_mul_f32");
+  return out;
+}
+
+void check_sig_caches(const at::Tensor& act, const at::Tensor& kc, const at::Tensor& vc, int G, int dim, int vdim) {
+  CHECK_CUDA(kc); CHECK_CUDA(vc); same_type(kc, act, "k_cache"); same_type(vc, act, "v_cache");
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous(), "caches must be contiguous 4-d");
+  TORCH_CHECK(kc.size(1) == G && kc.size(3) == dim && vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(2) == vdim &&
+              vc.size(3) == kc.size(2), "cache layout: K [NB, G, BS, dim], V [NB, G, vdim, BS]");
+  TORCH_CHECK(reinterpret_cast<uintptr_t>(kc.data_ptr()) % 16 == 0 && reinterpret_cast<uintptr_t>(vc.data_ptr()) % 16 == 0, "cache alignment");
+}
+
+void unitnorm_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64_t vdim, double eps, at::Tensor& kc,
+                       at::Tensor& vc, const at::Tensor& slots) {
+  CHECK_CUDA(qkv); CHECK_LASTDIM(qkv); CHECK_I32(slots); CHECK_CONTIG(slots);
+  const int esz = esz_of(qkv, "qkv");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) == (H + G) * dim + G * vdim, "qkv must be [T, (H + G) dim + G vdim]");
+  TORCH_CHECK(slots.numel() >= qkv.size(0), "slots");
+  check_sig_caches(qkv, kc, vc, G, dim, vdim);
+  const int BS = kc.size(2);
+  const long nslots = kc.size(0) * BS;
+  (void)nslots;
+  CHECK_RC(lk_unitnorm_kv_write(qkv.data_ptr(), qkv.stride(0), qkv.size(0), H, G, dim, vdim, (float)eps, kc.data_ptr(),
+                                vc.data_ptr(), ip(slots), BS, esz, cur_stream()), "unitnorm_kv_write");
+}
+
+at::Tensor sigattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt,
+                           const at::Tensor& cu_q, const at::Tensor& ctx, const at::Tensor& tile_seq,
+                           const at::Tensor& tile_q0, int64_t H, int64_t G, int64_t dim, int64_t vdim, double scale,
+                           const at::Tensor& r1, const at::Tensor& r2, const at::Tensor& pb, at::Tensor& out) {
+  CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_LASTDIM(out); same_type(out, q, "out");
+  const int esz = esz_of(q, "q");
+  check_sig_caches(q, kc, vc, G, dim, vdim);
+  CHECK_I32(bt); CHECK_I32(cu_q); CHECK_I32(ctx); CHECK_I32(tile_seq); CHECK_I32(tile_q0);
+  CHECK_CONTIG(cu_q); CHECK_CONTIG(ctx); CHECK_CONTIG(tile_seq); CHECK_CONTIG(tile_q0);
+  TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1 && bt.size(0) >= cu_q.numel() - 1 && ctx.numel() >= cu_q.numel() - 1, "block tables / ctx");
+  TORCH_CHECK(q.dim() == 2 && q.size(1) >= H * dim && out.dim() == 2 && out.size(0) >= q.size(0) && out.size(1) >= H * vdim, "q / out shape");
+  TORCH_CHECK(tile_seq.numel() == tile_q0.numel(), "tiles");
+  check_rows16(q, "q");
+  CHECK_RC(lk_sigattn_prefill(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), bt.stride(0), ip(cu_q), ip(ctx),
+                              ip(tile_seq), ip(tile_q0), tile_seq.numel(), H, G, dim, vdim, kc.size(2), (float)scale,
+                              fp(r1, H, "r1"), fp(r2, H, "r2"), fp(pb, H, "pb"), out.data_ptr(), out.stride(0), esz,
+                              cur_stream()), "sigattn_prefill");
+  return out;
+}
+
+at::Tensor sigattn_decode(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt,
+                          const at::Tensor& ctx, int64_t Z, int64_t H, int64_t G, int64_t dim, int64_t vdim, double scale,
+                          const at::Tensor& r1, const at::Tensor& r2, const at::Tensor& pb, at::Tensor& out,
+                          const c10::optional<at::Tensor>& part) {
+  CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_LASTDIM(out); same_type(out, q, "out");
+  const int esz = esz_of(q, "q");
+  check_sig_caches(q, kc, vc, G, dim, vdim);
+  CHECK_I32(bt); CHECK_I32(ctx); CHECK_CONTIG(ctx);
+  const long B = q.size(0);
+  TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1 && bt.size(0) >= B && ctx.numel() >= B, "block tables / ctx");
+  TORCH_CHECK(q.dim() == 2 && q.size(1) >= H * dim && out.dim() == 2 && out.size(0) >= B && out.size(1) >= H * vdim, "q / out shape");
+  TORCH_CHECK(Z >= 1 && Z <= 65535, "splits");
+  float* pp = nullptr;
+  if (Z > 1) {
+    TORCH_CHECK(part && part->is_cuda() && part->scalar_type() == at::kFloat && part->is_contiguous() &&
+                part->numel() >= B * H * Z * vdim, "part must be f32 [B, H, Z, vdim]");
+    pp = part->data_ptr<float>();
+  }
+  check_rows16(q, "q");
+  CHECK_RC(lk_sigattn_decode(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), bt.stride(0), ip(ctx), B, Z, H, G,
+                             dim, vdim, kc.size(2), (float)scale, fp(r1, H, "r1"), fp(r2, H, "r2"), fp(pb, H, "pb"),
+                             out.data_ptr(), out.stride(0), pp, esz, cur_stream()), "sigattn_decode");
+  return out;
+}
+
+void check_seqs(const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& positions, long rows) {
+  CHECK_CUDA(cu); CHECK_I32(cu); CHECK_I32(slots); CHECK_I32(positions);
+  CHECK_CONTIG(cu); CHECK_CONTIG(slots); CHECK_CONTIG(positions);
+  TORCH_CHECK(cu.numel() >= 2 && slots.numel() >= cu.numel() - 1 && positions.numel() >= rows, "cu / slots / positions");
+}
+
+// u: [T, >= col0 + C] rows of the input projection; the convolved channels are columns [col0, col0 + C)
+at::Tensor conv_silu(const at::Tensor& u, int64_t col0, int64_t C, const at::Tensor& w, const c10::optional<at::Tensor>& bias,
+                     at::Tensor& state, const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& positions,
+                     int64_t max_len) {
+  CHECK_CUDA(u); CHECK_LASTDIM(u);
+  const int esz = esz_of(u, "u");
+  TORCH_CHECK(u.dim() == 2 && col0 >= 0 && col0 + C <= u.size(1), "u columns");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C, "conv weight must be [C, taps]");
+  const int taps = w.size(1);
+  check_seqs(cu, slots, positions, u.size(0));
+  CHECK_CUDA(state); same_type(state, u, "conv state"); CHECK_CONTIG(state);
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == std::max(taps - 1, 1) && state.size(2) == C, "conv state must be [slots, taps - 1, C]");
+  TORCH_CHECK(max_len >= 1 && max_len <= u.size(0), "max_len");
+  at::Tensor out = at::empty({u.size(0), C}, u.options());
+  CHECK_RC(lk_conv_silu((const char*)u.data_ptr() + col0 * esz, u.stride(0), C, taps, fp(w, C * taps, "conv weight"),
+                        fpo(bias, C, "conv bias"), state.data_ptr(), ip(cu), ip(slots), ip(positions), cu.numel() - 1, max_len,
+                        out.data_ptr(), out.stride(0), esz, cur_stream()), "conv_silu");
+  return out;
+}
+
+// xbc: [T, heads P + 2 groups N] = [x | B | C] after the convolution; dt: [T, heads] view (row-strided)
+at::Tensor ssm_scan(const at::Tensor& xbc, const at::Tensor& dt, int64_t heads, int64_t P, int64_t N, int64_t groups,
+                    const at::Tensor& dt_bias, const at::Tensor& A_log, const at::Tensor& D, at::Tensor& state,
+                    const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& positions) {
+  CHECK_CUDA(xbc); CHECK_LASTDIM(xbc); CHECK_LASTDIM(dt);
+  const int esz = esz_of(xbc, "xbc");
+  same_type(dt, xbc, "dt");
+  TORCH_CHECK(xbc.dim() == 2 && xbc.size(1) == heads * P + 2 * groups * N && dt.dim() == 2 && dt.size(0) == xbc.size(0) && dt.size(1) == heads, "xbc / dt shape");
+  check_seqs(cu, slots, positions, xbc.size(0));
+  CHECK_CUDA(state); CHECK_F32(state); CHECK_CONTIG(state);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == P && state.size(3) == N, "state must be f32 [slots, heads, P, N]");
+  at::Tensor y = at::empty({xbc.size(0), heads * P}, xbc.options().dtype(at::kFloat));
+  CHECK_RC(lk_ssm_scan(xbc.data_ptr(), xbc.stride(0), dt.data_ptr(), dt.stride(0), cu.numel() - 1, heads, P, N, groups,
+                       fp(dt_bias, heads, "dt_bias"), fp(A_log, heads, "A_log"), fp(D, heads, "D"), state.data_ptr<float>(),
+                       ip(cu), ip(slots), ip(positions), y.data_ptr<float>(), y.stride(0), esz, cur_stream()), "ssm_scan");
+  return y;
+}
+
+at::Tensor gated_group_rmsnorm(const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t ngroups, double eps) {
+  CHECK_CUDA(y); CHECK_F32(y); CHECK_LASTDIM(y); CHECK_CUDA(z); CHECK_LASTDIM(z);
+  const int esz = esz_of(z, "z");
+  TORCH_CHECK(y.dim() == 2 && z.dim() == 2 && z.size(0) == y.size(0) && z.size(1) == y.size(1), "y / z shape");
+  const int inner = y.size(1);
+  at::Tensor out = at::empty({y.size(0), inner}, z.options());
+  CHECK_RC(lk_gated_group_rmsnorm(y.data_ptr<float>(), y.stride(0), z.data_ptr(), z.stride(0), fp(w, inner, "w"), y.size(0),
+                                  inner, ngroups, (float)eps, out.data_ptr(), out.stride(0), esz, cur_stream()),
+           "gated_group_rmsnorm");
+  return out;
+}
+
+}  // namespace
 // build provenance: "LKSTAMP:<hash of sources + flags>", generated by csrc/build.py at link time
 extern "C" const char lk_source_stamp[];
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("embed_pos", &embed_pos);
+  m.def("stream_embed_errors", []() { return lk_stream_embed_errors(); });
+  m.def("stream_rmsnorm", &stream_rmsnorm);
+  m.def("softcap", &softcap);
+  m.def("silu_mul_f32", &silu_mul_f32);
+  m.def("sigattn_supported", [](int64_t H, int64_t G, int64_t dim, int64_t vdim, int64_t BS, int64_t esz) {
+    return lk_sigattn_supported((int)H, (int)G, (int)dim, (int)vdim, (int)BS, (int)esz) != 0;
+  });
+  m.def("unitnorm_kv_write", &unitnorm_kv_write);
+  m.def("sigattn_prefill", &sigattn_prefill);
+  m.def("sigattn_decode", &sigattn_decode);
+  m.def("conv_silu", &conv_silu);
+  m.def("ssm_scan", &ssm_scan);
+  m.def("gated_group_rmsnorm", &gated_group_rmsnorm);
   m.def("window_mark", [](int64_t id) { CHECK_RC(lk_window_mark((int)id, cur_stream()), "window_mark"); });
   m.def("debug_invalid_launch", []() { CHECK_RC(lk_debug_invalid_launch(cur_stream()), "debug_invalid_launch"); });
   // a HIP stream restricted to the CUs of a bit mask (32 CUs per word): two kernels that

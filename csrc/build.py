@@ -29,6 +29,9 @@ BUILD = ROOT / "build" / "csrc"
 PKG = ROOT / "llm_kubernetes_minikube_sharp4dev_amd"
 ARCH = os.environ.get("LK_OFFLOAD_ARCH", "gfx950")
 EXT_NAME = "_C"
+# device code is generated without packed-f32 instructions (v_pk_add / mul / fma_f32): plain f32
+# code keeps its scalar VALU forms (the host pass warns that it does not know the feature)
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def _torch_paths():
@@ -62,8 +65,8 @@ def _codegen_flags(debug: bool = False) -> tuple[list[str], list[str]]:
     common = ["-O3", "-fPIC", "-std=c++17"]
     if debug:
         common += ["-DLK_DEBUG", "-g"]
-    kern = common + [f"--offload-arch={ARCH}", "-munsafe-fp-atomics", "-ffp-contract=fast"]
-    bind = common + [f"--offload-arch={ARCH}", "-DTORCH_API_INCLUDE_EXTENSION_H", f"-DTORCH_EXTENSION_NAME={EXT_NAME}",
+    kern = common + [f"--offload-arch={ARCH}", "-munsafe-fp-atomics", "-ffp-contract=fast", *NO_PACKED_FP32]
+    bind = common + [f"--offload-arch={ARCH}", *NO_PACKED_FP32, "-DTORCH_API_INCLUDE_EXTENSION_H", f"-DTORCH_EXTENSION_NAME={EXT_NAME}",
                      "-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1"]
     return kern, bind
 
@@ -102,9 +105,10 @@ def build(clean: bool = False, jobs: int | None = None, verbose: bool = False, d
     common = ["-O3", "-fPIC", "-std=c++17", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", f"-I{CSRC}"]
     if debug:
         common += ["-DLK_DEBUG", "-g"]
-    kern_flags = common + [f"--offload-arch={ARCH}", "-munsafe-fp-atomics", "-ffp-contract=fast"]
+    kern_flags = common + [f"--offload-arch={ARCH}", "-munsafe-fp-atomics", "-ffp-contract=fast", *NO_PACKED_FP32]
     bind_flags = common + [
         f"--offload-arch={ARCH}",
+        *NO_PACKED_FP32,
         "-DTORCH_API_INCLUDE_EXTENSION_H",
         f"-DTORCH_EXTENSION_NAME={EXT_NAME}",
         "-DUSE_ROCM=1",

@@ -216,3 +216,37 @@ int lk_embed_rows(bf16_t* out, const bf16_t* table, const int* ids, long T, int 
 int lk_embed_errors();  // out-of-table ids seen by strict lk_embed_rows since the last call
 int lk_scatter_ids(int* ids, const long* dst, const int* prev, const long* src, int n, hipStream_t st);
 int lk_gather_rows(bf16_t* out, const bf16_t* x, long xs, const long* idx, long R, int H, hipStream_t st);
+
+// csrc/stream_f32.hip: f32 residual stream (esz = element size of the bf16 / f32 activations)
+int lk_embed_pos(const int* ids, const int* positions, const void* tok, int vocab, const void* pos, int max_pos, long rows,
+                 int W, float* x, float* copy, int esz, hipStream_t st);
+int lk_stream_embed_errors();  // ids / positions outside their tables seen by lk_embed_pos (their rows are zero)
+int lk_stream_rmsnorm(float* x, const void* a, long as, const void* b, long bs, const float* e, float m, const float* w,
+                      float woff, float eps, const long* idx, long out_rows, void* out, long os, int W, int esz,
+                      hipStream_t st);
+int lk_silu_mul_f32(const float* x, long xs, float* out, long os, long rows, int I, hipStream_t st);
+int lk_softcap(const void* in, long is, float cap, float* out, long os, long rows, int V, int esz, hipStream_t st);
+
+// csrc/attn_sigmoid.hip: sigmoid attention with a log-distance penalty (K cache [NB, G, BS, dim], V cache
+// [NB, G, vdim, BS])
+int lk_sigattn_supported(int H, int G, int dim, int vdim, int BS, int esz);
+int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, float eps, void* kc, void* vc,
+                         const int* slots, int BS, int esz, hipStream_t st);
+int lk_sigattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride,
+                       const int* cu_q, const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H,
+                       int G, int dim, int vdim, int BS, float scale, const float* r1, const float* r2, const float* pb,
+                       void* out, long os, int esz, hipStream_t st);
+int lk_sigattn_decode(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride,
+                      const int* ctx_lens, int B, int Z, int H, int G, int dim, int vdim, int BS, float scale,
+                      const float* r1, const float* r2, const float* pb, void* out, long os, float* part, int esz,
+                      hipStream_t st);
+
+// csrc/ssm.hip: selective state-space mixer (sequences = rows [cu[s], cu[s+1]), state slot slots[s])
+int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const float* bias, void* state, const int* cu,
+                 const int* slots, const int* positions, int S, int max_len, void* out, long os, int esz,
+                 hipStream_t st);
+int lk_ssm_scan(const void* xbc, long xs, const void* dt, long dts, int S, int heads, int P, int N, int groups,
+                const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
+                const int* positions, float* y, long ys, int esz, hipStream_t st);
+int lk_gated_group_rmsnorm(const float* y, long ys, const void* z, long zs, const float* w, long rows, int inner,
+                           int ngroups, float eps, void* out, long os, int esz, hipStream_t st);

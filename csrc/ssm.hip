@@ -1,0 +1,277 @@
+// Mamba-2 style selective state-space mixer, token-parallel where it can be and sequential only
+// along the recurrence:
+//
+//   u_t  = [z | x B C | dt]                       the input projection's row (bf16 or f32)
+//   xBC  = silu(causal_conv(x B C) + b)           per channel, `taps` wide, the last column is the
+//                                                 current token's; the taps - 1 inputs before a chunk
+//                                                 come from the sequence's conv state
+//   dt   = softplus(dt + dt_bias)                 f32, no clamp
+//   S_t  = exp(-exp(A_log) dt) S_{t-1} + dt B_t x_t^T      S: [N, P] per head, f32, carried per sequence
+//   y_t  = S_t^T C_t + D x_t                      f32
+//   out  = groupRMS(y * silu(z)) * w              the gate comes before the norm
+//
+// A batch is a list of sequences (prefill chunks of any length, decode rows of length 1): rows
+// [cu[s], cu[s+1]) belong to sequence s, whose state lives in slot slots[s] (< 0: a padding row,
+// skipped) and starts from zero when its first row sits at position 0.
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+template <typename T>
+LK_DEVICE float ldf(const T* p);
+template <>
+LK_DEVICE float ldf<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <>
+LK_DEVICE float ldf<float>(const float* p) { return *p; }
+template <typename T>
+LK_DEVICE void stf(T* p, float v);
+template <>
+LK_DEVICE void stf<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+template <>
+LK_DEVICE void stf<float>(float* p, float v) { *p = v; }
+
+constexpr int kMaxTaps = 8;
+constexpr int kConvRows = 16;  // tokens per workgroup of the convolution
+
+template <bool EXACT>
+LK_DEVICE float silu_f(float x) {
+  if constexpr (EXACT) return x / (1.f + expf(-x));
+  else return x * __builtin_amdgcn_rcpf(1.f + __expf(-x));
+}
+
+// grid (sequence, token tile, channel block): out[row][c] = silu(sum_k w[c][k] in(i - (taps-1) + k) + b[c])
+template <typename T>
+__global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ u, long us, int C, int taps,
+                                                        const float* __restrict__ w, const float* __restrict__ bias,
+                                                        const T* __restrict__ state, const int* __restrict__ cu,
+                                                        const int* __restrict__ slots,
+                                                        const int* __restrict__ positions, T* __restrict__ out,
+                                                        long os) {
+  const int s = blockIdx.x, c = blockIdx.z * 256 + threadIdx.x;
+  const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
+  const int i0 = blockIdx.y * kConvRows;
+  if (c >= C || i0 >= len) return;
+  if (slot < 0) {
+    for (int i = i0; i < min(len, i0 + kConvRows); ++i) stf<T>(out + (long)(row0 + i) * os + c, 0.f);
+    return;
+  }
+  const bool past = positions[row0] > 0;
+  const T* st = state + (long)slot * (taps - 1) * C + c;
+  float wk[kMaxTaps];
+#pragma unroll
+  for (int k = 0; k < kMaxTaps; ++k) wk[k] = k < taps ? w[(long)c * taps + k] : 0.f;
+  const float b = bias ? bias[c] : 0.f;
+  for (int i = i0; i < min(len, i0 + kConvRows); ++i) {
+    float acc = b;
+#pragma unroll
+    for (int k = 0; k < kMaxTaps; ++k) {
+      if (k < taps) {
+        const int idx = i - (taps - 1) + k;
+        float v = 0.f;
+        if (idx >= 0) v = ldf<T>(u + (long)(row0 + idx) * us + c);
+        else if (past) v = ldf<T>(st + (long)(taps - 1 + idx) * C);
+        acc += wk[k] * v;
+      }
+    }
+    stf<T>(out + (long)(row0 + i) * os + c, silu_f<sizeof(T) == 4>(acc));
+  }
+}
+
+// grid (sequence, channel block): the sequence's last taps - 1 inputs become its conv state.
+// Runs after conv_silu_kernel (which reads the old state).
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(const T* __restrict__ u, long us, int C, int taps,
+                                                         T* __restrict__ state, const int* __restrict__ cu,
+                                                         const int* __restrict__ slots,
+                                                         const int* __restrict__ positions) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
+  if (c >= C || slot < 0 || len <= 0) return;
+  const bool past = positions[row0] > 0;
+  T* st = state + (long)slot * (taps - 1) * C + c;
+  T keep[kMaxTaps];
+#pragma unroll
+  for (int i = 0; i < kMaxTaps; ++i) {
+    if (i < taps - 1) {
+      const int idx = len - (taps - 1) + i;
+      T v;
+      stf<T>(&v, 0.f);
+      if (idx >= 0) v = u[(long)(row0 + idx) * us + c];
+      else if (past) v = st[(long)(i + len) * C];
+      keep[i] = v;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxTaps; ++i)
+    if (i < taps - 1) st[(long)i * C] = keep[i];
+}
+
+// Sequential scan.  grid (sequence, head, P / 16): 256 threads = 16 state columns p x 16 slices of
+// the N state rows (thread holds rows ns, ns + 16, ...), so y_t[p] is a 16-lane butterfly.
+// The next token's operands are fetched while the current one is applied.
+template <typename T, int NR>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc, long xs, const T* __restrict__ dtp,
+                                                       long dts, int heads, int P, int N, int groups,
+                                                       const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ A_log, const float* __restrict__ Dp,
+                                                       float* __restrict__ state, const int* __restrict__ cu,
+                                                       const int* __restrict__ slots,
+                                                       const int* __restrict__ positions, float* __restrict__ y,
+                                                       long ys) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int ns = threadIdx.x & 15, p = blockIdx.z * 16 + (threadIdx.x >> 4);
+  const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
+  if (len <= 0) return;
+  const bool pv = p < P;
+  if (slot < 0) {
+    if (pv && ns == 0)
+      for (int i = 0; i < len; ++i) y[(long)(row0 + i) * ys + (long)h * P + p] = 0.f;
+    return;
+  }
+  const int inner = heads * P, grp = h / (heads / groups);
+  const long xo = (long)h * P + (pv ? p : 0), bo = inner + (long)grp * N, co = inner + (long)groups * N + (long)grp * N;
+  float* sp = state + (((long)slot * heads + h) * P + (pv ? p : 0)) * N;
+  float S[NR];
+  const bool past = positions[row0] > 0;
+#pragma unroll
+  for (int i = 0; i < NR; ++i) {
+    const int n = ns + 16 * i;
+    S[i] = (past && pv && n < N) ? sp[n] : 0.f;
+  }
+  const float nA = -expf(A_log[h]), db = dt_bias[h], Dh = Dp[h];
+  float Bn[NR], Cn[NR], xv, dtr;
+  auto fetch = [&](int i, float (&B)[NR], float (&Cc)[NR], float& x, float& d) {
+    const T* r = xbc + (long)(row0 + i) * xs;
+    x = ldf<T>(r + xo);
+    d = ldf<T>(dtp + (long)(row0 + i) * dts + h);
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      const int n = ns + 16 * k;
+      B[k] = n < N ? ldf<T>(r + bo + n) : 0.f;
+      Cc[k] = n < N ? ldf<T>(r + co + n) : 0.f;
+    }
+  };
+  fetch(0, Bn, Cn, xv, dtr);
+  for (int i = 0; i < len; ++i) {
+    float B[NR], Cc[NR];
+    const float x = xv, dr = dtr;
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      B[k] = Bn[k];
+      Cc[k] = Cn[k];
+    }
+    if (i + 1 < len) fetch(i + 1, Bn, Cn, xv, dtr);
+    const float a = dr + db;
+    const float dt = a > 20.f ? a : log1pf(expf(a));
+    const float dA = expf(nA * dt), dx = dt * x;
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      S[k] = dA * S[k] + dx * B[k];
+      acc += S[k] * Cc[k];
+    }
+    acc += __shfl_xor(acc, 1, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    acc += __shfl_xor(acc, 4, 64);
+    acc += __shfl_xor(acc, 8, 64);
+    if (pv && ns == 0) y[(long)(row0 + i) * ys + (long)h * P + p] = acc + Dh * x;
+  }
+  if (pv) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int n = ns + 16 * i;
+      if (n < N) sp[n] = S[i];
+    }
+  }
+}
+
+// grid (row, norm group): out = (y * silu(z)) / sqrt(mean_group((y silu z)^2) + eps) * w
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* __restrict__ y, long ys,
+                                                                  const T* __restrict__ z, long zs,
+                                                                  const float* __restrict__ w, int gs, float eps,
+                                                                  T* __restrict__ out, long os) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  const int c0 = blockIdx.y * gs;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < gs; c += 256) {
+    const float v = y[row * ys + c0 + c] * silu_f<sizeof(T) == 4>(ldf<T>(z + row * zs + c0 + c));
+    ss += v * v;
+  }
+  ss = block_sum<4>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)gs + eps);
+  for (int c = threadIdx.x; c < gs; c += 256) {
+    const float v = y[row * ys + c0 + c] * silu_f<sizeof(T) == 4>(ldf<T>(z + row * zs + c0 + c));
+    stf<T>(out + row * os + c0 + c, v * inv * w[c0 + c]);
+  }
+}
+
+template <typename T>
+int scan_t(const T* xbc, long xs, const T* dtp, long dts, int S, int heads, int P, int N, int groups,
+           const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
+           const int* positions, float* y, long ys, hipStream_t st) {
+  dim3 grid(S, heads, (P + 15) / 16);
+#define LK_SCAN(NR)                                                                                                 \
+  ssm_scan_kernel<T, NR><<<grid, 256, 0, st>>>(xbc, xs, dtp, dts, heads, P, N, groups, dt_bias, A_log, D, state, cu, \
+                                               slots, positions, y, ys)
+  if (N <= 16) LK_SCAN(1);
+  else if (N <= 32) LK_SCAN(2);
+  else if (N <= 64) LK_SCAN(4);
+  else if (N <= 128) LK_SCAN(8);
+  else if (N <= 256) LK_SCAN(16);
+  else return -1;
+#undef LK_SCAN
+  LK_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // namespace
+
+int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const float* bias, void* state, const int* cu,
+                 const int* slots, const int* positions, int S, int max_len, void* out, long os, int esz,
+                 hipStream_t st) {
+  if (S <= 0 || max_len <= 0) return 0;
+  if (taps < 1 || taps > kMaxTaps || C <= 0) return -1;
+  dim3 grid(S, (max_len + kConvRows - 1) / kConvRows, (C + 255) / 256), g2(S, (C + 255) / 256);
+  if (esz == 2) {
+    conv_silu_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)u, us, C, taps, w, bias, (const bf16_t*)state, cu,
+                                                   slots, positions, (bf16_t*)out, os);
+    LK_CHECK_LAUNCH();
+    if (taps > 1) conv_state_kernel<bf16_t><<<g2, 256, 0, st>>>((const bf16_t*)u, us, C, taps, (bf16_t*)state, cu, slots, positions);
+  } else {
+    conv_silu_kernel<float><<<grid, 256, 0, st>>>((const float*)u, us, C, taps, w, bias, (const float*)state, cu, slots,
+                                                  positions, (float*)out, os);
+    LK_CHECK_LAUNCH();
+    if (taps > 1) conv_state_kernel<float><<<g2, 256, 0, st>>>((const float*)u, us, C, taps, (float*)state, cu, slots, positions);
+  }
+  LK_CHECK_LAUNCH();
+  return 0;
+}
+
+int lk_ssm_scan(const void* xbc, long xs, const void* dt, long dts, int S, int heads, int P, int N, int groups,
+                const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
+                const int* positions, float* y, long ys, int esz, hipStream_t st) {
+  if (S <= 0) return 0;
+  if (heads <= 0 || groups <= 0 || heads % groups || P <= 0 || N <= 0) return -1;
+  return esz == 2 ? scan_t<bf16_t>((const bf16_t*)xbc, xs, (const bf16_t*)dt, dts, S, heads, P, N, groups, dt_bias,
+                                   A_log, D, state, cu, slots, positions, y, ys, st)
+                  : scan_t<float>((const float*)xbc, xs, (const float*)dt, dts, S, heads, P, N, groups, dt_bias, A_log,
+                                  D, state, cu, slots, positions, y, ys, st);
+}
+
+int lk_gated_group_rmsnorm(const float* y, long ys, const void* z, long zs, const float* w, long rows, int inner,
+                           int ngroups, float eps, void* out, long os, int esz, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (ngroups <= 0 || inner % ngroups) return -1;
+  dim3 grid((unsigned)rows, ngroups);
+  if (esz == 2)
+    gated_group_rmsnorm_kernel<bf16_t><<<grid, 256, 0, st>>>(y, ys, (const bf16_t*)z, zs, w, inner / ngroups, eps,
+                                                             (bf16_t*)out, os);
+  else
+    gated_group_rmsnorm_kernel<float><<<grid, 256, 0, st>>>(y, ys, (const float*)z, zs, w, inner / ngroups, eps,
+                                                            (float*)out, os);
+  LK_CHECK_LAUNCH();
+  return 0;
+}

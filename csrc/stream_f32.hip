@@ -1,0 +1,153 @@
+// A residual stream kept in f32 next to bf16 (or f32) sublayer outputs:
+//   * token + learned position embedding gather into the f32 stream (and a second copy for models
+//     that add the embedding output again later);
+//   * fused "stream update + RMSNorm": x += m * (a + b) + e, h = x / sqrt(mean(x^2) + eps) * (off + w)
+//     -- the update of a block whose sublayers all read one norm's output and are summed, and the
+//     next block's norm, in one pass over the row (a, b, e optional; off = 1 for weights stored
+//     around zero); with a row index list it gathers rows instead and leaves the stream alone (the
+//     rows that feed the LM head);
+//   * soft-capped logits: cap * tanh(z / cap), f32 out.
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+template <typename T>
+LK_DEVICE float ldv(const T* p);
+template <>
+LK_DEVICE float ldv<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <>
+LK_DEVICE float ldv<float>(const float* p) { return *p; }
+template <typename T>
+LK_DEVICE void stv(T* p, float v);
+template <>
+LK_DEVICE void stv<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+template <>
+LK_DEVICE void stv<float>(float* p, float v) { *p = v; }
+
+__device__ int g_stream_embed_errors = 0;
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_pos_kernel(const int* __restrict__ ids, const int* __restrict__ positions,
+                                                        const T* __restrict__ tok, int vocab,
+                                                        const T* __restrict__ pos, int max_pos, int W,
+                                                        float* __restrict__ x, float* __restrict__ copy) {
+  const long row = blockIdx.x;
+  const int id = ids[row], ps = positions[row];
+  const bool ok = id >= 0 && id < vocab && ps >= 0 && ps < max_pos;
+  if (!ok && threadIdx.x == 0) atomicAdd(&g_stream_embed_errors, 1);
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = ok ? ldv<T>(tok + (long)id * W + c) + ldv<T>(pos + (long)ps * W + c) : 0.f;
+    x[row * W + c] = v;
+    if (copy) copy[row * W + c] = v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void stream_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ a, long as,
+                                                             const T* __restrict__ b, long bs,
+                                                             const float* __restrict__ e, float m,
+                                                             const float* __restrict__ w, float woff, float eps,
+                                                             const long* __restrict__ idx, T* __restrict__ out, long os,
+                                                             int W) {
+  __shared__ float red[4];
+  const long orow = blockIdx.x, row = idx ? idx[orow] : orow;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float v = x[row * W + c];
+    float d = 0.f;
+    if (a) d += ldv<T>(a + row * as + c);
+    if (b) d += ldv<T>(b + row * bs + c);
+    v += m * d;
+    if (e) v += e[row * W + c];
+    if (!idx && (a || b || e)) x[row * W + c] = v;
+    ss += v * v;
+  }
+  ss = block_sum<4>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float v;
+    if (!idx) {
+      v = x[row * W + c];  // this thread's own store above (or the untouched stream)
+    } else {
+      v = x[row * W + c];
+      float d = 0.f;
+      if (a) d += ldv<T>(a + row * as + c);
+      if (b) d += ldv<T>(b + row * bs + c);
+      v += m * d;
+      if (e) v += e[row * W + c];
+    }
+    stv<T>(out + orow * os + c, v * inv * (w ? woff + w[c] : 1.f));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softcap_kernel(const T* __restrict__ in, long is, float cap, float* __restrict__ out,
+                                                      long os, int V) {
+  const long row = blockIdx.x;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < V; c += 256 * gridDim.y) {
+    const float z = ldv<T>(in + row * is + c);
+    out[row * os + c] = cap > 0.f ? cap * tanhf(z / cap) : z;
+  }
+}
+
+// out[r][c] = silu(x[r][c]) * x[r][I + c] for f32 rows [gate | up] (the bf16 case is the GEMM's epilogue)
+__global__ __launch_bounds__(256) void silu_mul_f32_kernel(const float* __restrict__ x, long xs, float* __restrict__ out,
+                                                           long os, int I) {
+  const long row = blockIdx.x;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < I; c += 256 * gridDim.y) {
+    const float g = x[row * xs + c];
+    out[row * os + c] = g / (1.f + expf(-g)) * x[row * xs + I + c];
+  }
+}
+
+}  // namespace
+
+int lk_silu_mul_f32(const float* x, long xs, float* out, long os, long rows, int I, hipStream_t st) {
+  if (rows <= 0) return 0;
+  silu_mul_f32_kernel<<<dim3((unsigned)rows, (unsigned)((I + 2047) / 2048)), 256, 0, st>>>(x, xs, out, os, I);
+  LK_CHECK_LAUNCH();
+  return 0;
+}
+
+int lk_stream_embed_errors() {
+  int v = 0;
+  if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_stream_embed_errors), sizeof(int)) != hipSuccess) return -1;
+  return v;
+}
+
+int lk_embed_pos(const int* ids, const int* positions, const void* tok, int vocab, const void* pos, int max_pos, long rows,
+                 int W, float* x, float* copy, int esz, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (esz == 2)
+    embed_pos_kernel<bf16_t><<<(unsigned)rows, 256, 0, st>>>(ids, positions, (const bf16_t*)tok, vocab, (const bf16_t*)pos,
+                                                             max_pos, W, x, copy);
+  else
+    embed_pos_kernel<float><<<(unsigned)rows, 256, 0, st>>>(ids, positions, (const float*)tok, vocab, (const float*)pos,
+                                                            max_pos, W, x, copy);
+  LK_CHECK_LAUNCH();
+  return 0;
+}
+
+int lk_stream_rmsnorm(float* x, const void* a, long as, const void* b, long bs, const float* e, float m, const float* w,
+                      float woff, float eps, const long* idx, long out_rows, void* out, long os, int W, int esz,
+                      hipStream_t st) {
+  if (out_rows <= 0) return 0;
+  if (esz == 2)
+    stream_rmsnorm_kernel<bf16_t><<<(unsigned)out_rows, 256, 0, st>>>(x, (const bf16_t*)a, as, (const bf16_t*)b, bs, e, m, w,
+                                                                      woff, eps, idx, (bf16_t*)out, os, W);
+  else
+    stream_rmsnorm_kernel<float><<<(unsigned)out_rows, 256, 0, st>>>(x, (const float*)a, as, (const float*)b, bs, e, m, w,
+                                                                     woff, eps, idx, (float*)out, os, W);
+  LK_CHECK_LAUNCH();
+  return 0;
+}
+
+int lk_softcap(const void* in, long is, float cap, float* out, long os, long rows, int V, int esz, hipStream_t st) {
+  if (rows <= 0) return 0;
+  dim3 grid((unsigned)rows, (unsigned)((V + 2047) / 2048));
+  if (esz == 2) softcap_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)in, is, cap, out, os, V);
+  else softcap_kernel<float><<<grid, 256, 0, st>>>((const float*)in, is, cap, out, os, V);
+  LK_CHECK_LAUNCH();
+  return 0;
+}

@@ -544,6 +544,13 @@ def cmd_router(args):
     _uvicorn(create_router_app(args.backends.split(",")), args.host, args.port)
 
 
+def cmd_trace_run(args):
+    from .engine.replay import run_trace
+
+    return run_trace(args.model, args.dtype, args.out, args.max_tokens, max_seqs=args.max_seqs, device=args.device,
+                     use_graphs=not args.no_graphs)
+
+
 def _tp_args(p):
     p.add_argument("--tp", type=int, default=None,
                    help="(default: engine.tp_size of the config, 1) tensor-parallel degree: the generator's weights / KV heads / vocab and the RAG corpus "
@@ -641,6 +648,16 @@ def main(argv=None):
     p.add_argument("--fault-rate", type=float, default=0.0)
     p.add_argument("--latency", type=float, default=0.0)
     p.set_defaults(fn=cmd_fake_apiserver)
+    p = sub.add_parser("trace-run", help="replay given token ids step by step (JSON lines on stdin) and write logits")
+    p.add_argument("--model", required=True, help="checkpoint directory (config.json + *.safetensors)")
+    p.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    p.add_argument("--out", required=True, help="directory for <step>.f32")
+    p.add_argument("--max-tokens", type=int, required=True, help="cache pool size in tokens (live requests)")
+    p.add_argument("--max-seqs", type=int, default=4, help="state slots / live requests")
+    p.add_argument("--device", default="auto")
+    p.add_argument("--no-graphs", action="store_true", help="do not capture decode steps in hipGraphs")
+    p.set_defaults(fn=cmd_trace_run)
+
     p = common(sub.add_parser("router"), 11434)
     p.add_argument("--backends", required=True)
     p.set_defaults(fn=cmd_router)

@@ -111,6 +111,39 @@ class BlockAllocator:
         return h
 
 
+class NoFreeSlots(RuntimeError):
+    pass
+
+
+class StateSlotPool:
+    """Fixed-size per-sequence state slots (recurrent / convolution state of stateful mixers): a
+    running sequence holds one slot from admission until it finishes or is preempted; a freed slot
+    is handed out again (lowest id first) and its new owner starts from a zero state because its
+    first token sits at position 0, not because anything is cleared here."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free = list(range(num_slots - 1, -1, -1))
+        self._held: set = set()
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def acquire(self) -> int:
+        if not self._free:
+            raise NoFreeSlots()
+        s = self._free.pop()
+        self._held.add(s)
+        return s
+
+    def release(self, slot: int):
+        if slot in self._held:
+            self._held.remove(slot)
+            self._free.append(slot)
+            self._free.sort(reverse=True)
+
+
 def make_allocator(num_blocks: int, block_size: int, prefix_caching: bool = True, prefer_native: bool = True):
     if prefer_native:
         try:

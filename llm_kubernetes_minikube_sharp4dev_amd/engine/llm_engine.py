@@ -15,7 +15,7 @@ import torch
 
 from ..utils import metrics as M
 from ..utils.logging import get_logger
-from .block_manager import make_allocator
+from .block_manager import StateSlotPool, make_allocator
 from .model_runner import ModelRunner
 from .sampling import Sampler, SamplingParams
 from .scheduler import Scheduler
@@ -70,7 +70,12 @@ class LLMEngine:
         self.tokenizer = tokenizer
         self.runner = _runner or ModelRunner(model, block_size, max_model_len, max_num_seqs, num_blocks,
                                              kv_cache_gb, gpu_memory_fraction, use_graphs)
-        self.allocator = make_allocator(self.runner.num_blocks, block_size, enable_prefix_caching)
+        # a stateful model (recurrent mixers) cannot reuse another request's cached blocks: the
+        # state after the shared prefix is not kept.  Its sequences hold a state slot while they run.
+        stateful = bool(getattr(model, "stateful", False))
+        self.allocator = make_allocator(self.runner.num_blocks, block_size, enable_prefix_caching and not stateful)
+        self.state_pool = StateSlotPool(max_num_seqs) if stateful else None
+        self._replay: dict = {}  # replay_step: request id -> its sequence
         if prefill_hold is None:
             # new prefill waits up to 4 steps for a full 4096-token step while >= 64 decode rows keep
             # the GPU busy: the prefill GEMMs cost ~10 % less per row at 4,096 rows than at ~2,500
@@ -81,7 +86,8 @@ class LLMEngine:
                                    token_align, token_align_wave, prefill_hold,
                                    int(os.environ.get("LK_HOLD_MIN_DECODE", "64")),
                                    float(os.environ.get("LK_HOLD_FILL", "1.0")),
-                                   _small_buckets(), int(os.environ.get("LK_HOLD_SMALL", "0")))
+                                   _small_buckets(), int(os.environ.get("LK_HOLD_SMALL", "0")),
+                                   state_pool=self.state_pool)
         self.sampler = Sampler(model.cfg.vocab_size, seed, history_len=max_model_len)
         self.max_model_len = max_model_len
         if eos_ids is None:
@@ -197,6 +203,60 @@ class LLMEngine:
             p, self._pending = self._pending, None
             out += self._collect(self._sample(p))
         return out
+
+    @torch.inference_mode()
+    def replay_step(self, entries: list, end=()) -> Optional[torch.Tensor]:
+        """One engine step over GIVEN tokens instead of sampled ones (trace replay, scoring):
+        ``entries`` = [(request id, its next tokens, offsets among them whose logits are wanted)];
+        a request is admitted at its first entry (these tokens are its prompt; later entries are
+        appended like generated tokens, so a one-token entry is a decode row and longer ones are
+        prefill chunks) and may sit out any number of steps.  All entries run as one batch through
+        the model runner, the block allocator and the state pool that generation uses.  ``end``:
+        requests finished after this step (their blocks and state slot are freed).
+        Returns f32 logits [wanted rows, vocab] in the order of the entries and their offsets
+        (None if nothing is wanted).  Raises if the cache pool or the state slots cannot hold the
+        live requests (replay never preempts)."""
+        with self.lock:
+            items, want = [], {}
+            for rid, toks, offs in entries:
+                toks = [int(t) for t in toks]
+                if not toks:
+                    continue
+                seq = self._replay.get(rid)
+                if seq is None:
+                    seq = self._replay[rid] = Sequence(toks, SamplingParams(max_tokens=1 << 30))
+                    seq.req_id = rid
+                else:
+                    seq.output_ids.extend(toks)
+                if seq.length > self.max_model_len:
+                    raise ValueError(f"request {rid}: {seq.length} tokens exceed max_model_len={self.max_model_len}")
+                if any(not 0 <= int(o) < len(toks) for o in offs):
+                    raise ValueError(f"request {rid}: a wanted offset lies outside its {len(toks)} tokens")
+                if not self.scheduler.admit_forced(seq, seq.length):
+                    raise RuntimeError(f"request {rid}: no cache blocks or state slot left for {seq.length} tokens")
+                items.append((seq, seq.num_computed, len(toks)))
+                want[id(seq)] = [int(o) for o in offs]
+            out = None
+            if items:
+                rows, lg = self.runner.forward_logits(items, False, want=want)
+                for seq, start, n in items:
+                    seq.num_computed = start + n
+                self.launches += 1
+                self.steps += 1
+                if rows:
+                    # the runner orders a step [prompt chunks | decode rows]: back to the entries' order
+                    at = {}
+                    for k, (seq, _) in enumerate(rows):
+                        at.setdefault(id(seq), []).append(k)
+                    order = [k for seq, _, _ in items for k in at.get(id(seq), [])]
+                    lg = lg.float()
+                    out = lg if order == list(range(len(order))) else lg.index_select(
+                        0, torch.tensor(order, dtype=torch.long, device=lg.device))
+            for rid in end:
+                seq = self._replay.pop(rid, None)
+                if seq is not None:
+                    self.scheduler.finish(seq, "stop")
+            return out
 
     def _launch(self):
         with self.lock:

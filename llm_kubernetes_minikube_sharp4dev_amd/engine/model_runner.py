@@ -104,8 +104,15 @@ class ModelRunner:
             num_blocks = self.plan_num_blocks(model, block_size, max_model_len, max_num_seqs, kv_cache_gb,
                                               gpu_memory_fraction)
         self.num_blocks = num_blocks
-        self.kv = torch.empty((self.L, 2, num_blocks, self.hkv, block_size, self.D), dtype=dt, device=self.device)
-        self.kv_caches = [(self.kv[l, 0], self.kv[l, 1]) for l in range(self.L)]
+        # stateful models (recurrent mixers) also get max_num_seqs state slots and tell the step which
+        # slot each of its sequences holds; such a model lays out its own caches (one per layer run)
+        self.stateful = bool(getattr(model, "stateful", False))
+        if hasattr(model, "make_caches"):
+            self.kv = None
+            self.kv_caches = model.make_caches(num_blocks, block_size, max_num_seqs)
+        else:
+            self.kv = torch.empty((self.L, 2, num_blocks, self.hkv, block_size, self.D), dtype=dt, device=self.device)
+            self.kv_caches = [(self.kv[l, 0], self.kv[l, 1]) for l in range(self.L)]
         log.info("kv cache: %d blocks x %d tokens (%.1f GB)", num_blocks, block_size,
                  num_blocks * block_bytes / 2**30)
         self.use_graphs = use_graphs and self.device.type == "cuda"
@@ -196,6 +203,8 @@ class ModelRunner:
 
     @staticmethod
     def block_bytes(model, block_size: int) -> int:
+        if hasattr(model, "cache_block_bytes"):
+            return max(1, model.cache_block_bytes(block_size))
         esz = torch.tensor([], dtype=model.dtype).element_size()
         return model.cfg.num_layers * 2 * model.hkv * block_size * model.D * esz
 
@@ -292,11 +301,19 @@ class ModelRunner:
         return bt
 
     # ----------------------------------------------------------- step inputs (host)
-    def prepare(self, items, greedy: bool = False):
+    def prepare(self, items, greedy: bool = False, want: Optional[dict] = None):
         """items [(seq, start, n)] -> (StepInputs of host arrays, rows [(seq, row)]).
         Everything a rank needs to run the step; a TP driver broadcasts it.  ``greedy``:
-        the step returns token ids (distributed argmax under TP) instead of logits."""
-        si, rows = self._prepare(items)
+        the step returns token ids (distributed argmax under TP) instead of logits.
+        ``want`` {id(seq): offsets within its chunk}: the rows whose logits the step returns, instead
+        of the last row of every sequence that has reached its end (replay of given tokens)."""
+        si, rows = self._prepare(items, want)
+        if self.stateful:
+            pre = [it for it in items if not self._as_decode(*it)] if not si.decode_graph else []
+            dec = [it for it in items if self._as_decode(*it)] if not si.decode_graph else items
+            sl = [s.state_slot for s, _, _ in pre] + [s.state_slot for s, _, _ in dec]
+            sl += [-1] * (max(si.decode_graph, 0) - len(sl))
+            si.state_slots = np.asarray(sl, dtype=np.int32)
         si.greedy = bool(greedy)
         if si.num_decode:  # keys the decode attention reads this step (in-situ bandwidth accounting)
             self.decode_kv_keys += int(np.asarray(si.ctx_d[: si.num_decode], dtype=np.int64).sum())
@@ -322,12 +339,21 @@ class ModelRunner:
         whose few query rows each walk the whole context in one workgroup."""
         if seq.is_decode:
             return True
+        if self.stateful:
+            return False  # a recurrent state advances one token at a time: chunks run as prefill
         return 1 < n <= EXTEND_AS_DECODE and start >= len(seq.prompt_ids) and seq.num_inflight == 0
 
-    def _prepare(self, items):
+    @staticmethod
+    def _rows_of(seq, start: int, n: int, first_row: int, want: Optional[dict]) -> list:
+        """Step rows of this chunk (first at ``first_row``) whose logits are returned."""
+        if want is not None:
+            return [(seq, first_row + int(o)) for o in want.get(id(seq), ())]
+        return [(seq, first_row + n - 1)] if start + n == seq.length + seq.num_inflight else []
+
+    def _prepare(self, items, want: Optional[dict] = None):
         if (self.use_graphs and items and all(self._as_decode(*it) for it in items)
                 and sum(n for _, _, n in items) <= self.graph_sizes[-1]):
-            return self._prepare_graph(items)
+            return self._prepare_graph(items, want)
         pre = [it for it in items if not self._as_decode(*it)]
         dec = [it for it in items if self._as_decode(*it)]
         ids, pos, slots = [], [], []
@@ -342,9 +368,8 @@ class ModelRunner:
             q_lens.append(n)
             ctx.append(start + n)
             tables.append(seq.block_table)
+            rows += self._rows_of(seq, start, n, r, want)
             r += n
-            if start + n == seq.length + seq.num_inflight:
-                rows.append((seq, r - 1))
         ctx_d = tables_d = None
         if dec:
             d_ids, d_pos, d_slots, ctx_d, tables_d = self._decode_rows(
@@ -353,9 +378,8 @@ class ModelRunner:
             pos.append(d_pos)
             slots.append(d_slots)
             for seq, start, n in dec:
+                rows += self._rows_of(seq, start, n, r, want)
                 r += n
-                if start + n == seq.length + seq.num_inflight:
-                    rows.append((seq, r - 1))
         nd = len(ctx_d) if dec else 0
         shared = self._shared_len(tables_d, ctx_d, nd) if dec else 0
         si = StepInputs(decode_graph=0, ids=np.asarray(ids, dtype=np.int32), positions=np.concatenate(pos),
@@ -366,7 +390,7 @@ class ModelRunner:
                         gather=self._gather(dec, r - nd) if dec else None, shared_len=shared)
         return si, rows
 
-    def _prepare_graph(self, items):
+    def _prepare_graph(self, items, want: Optional[dict] = None):
         """Decode rows (one-token steps and short extend chunks, expanded to causal rows)
         for the hipGraph of the smallest bucket that holds them; the graph computes every
         row's logits, the step keeps the rows that end a sequence's new tokens."""
@@ -375,9 +399,8 @@ class ModelRunner:
         ids, pos, slots, ctx, bt = self._decode_rows(items, self.max_blocks, Bg)
         rows, r = [], 0
         for seq, start, n in items:
+            rows += self._rows_of(seq, start, n, r, want)
             r += n
-            if start + n == seq.length + seq.num_inflight:
-                rows.append((seq, r - 1))
         si = StepInputs(decode_graph=Bg, ids=ids, positions=pos, slots=slots, ctx_d=ctx, tables_d=bt,
                         num_decode=B, logits_rows=np.asarray([row for _, row in rows], dtype=np.int64),
                         gather=self._gather(items, 0), shared_len=self._shared_len(bt, ctx, B))
@@ -422,6 +445,11 @@ class ModelRunner:
             host["logits"] = si.logits_rows
         if si.gather is not None:
             host.update(g_dst=si.gather[0], g_src=si.gather[1])
+        if si.state_slots is not None:
+            lens = list(si.q_lens) + [1] * si.num_decode
+            seq_cu = np.zeros(len(lens) + 1, dtype=np.int32)
+            seq_cu[1:] = np.cumsum(lens)
+            host.update(seq_cu=seq_cu, state_slots=si.state_slots)
         d = self._upload(host)
         meta = AttnMeta(positions=d["pos"], slots=d["slots"], num_prefill_tokens=Tp,
                         num_prefill_seqs=len(si.q_lens), num_decode=si.num_decode)
@@ -439,6 +467,9 @@ class ModelRunner:
             if "ts_u" in d:
                 meta.tiles_u = (d["ts_u"], d["tq_u"])
         meta.logits_idx = d.get("logits")
+        if si.state_slots is not None:
+            meta.seq_cu, meta.state_slots = d["seq_cu"], d["state_slots"]
+            meta.max_seq_len = max(list(si.q_lens) + [1])
         ids = d["ids"]
         if si.gather is not None:
             self._apply_gather(ids, d["g_dst"], d["g_src"])
@@ -495,12 +526,12 @@ class ModelRunner:
             buf = torch.empty(si.prev_bcast, dtype=torch.int32, device=self.device)
         self.prev_ids = tp.broadcast_(buf)
 
-    def forward_logits(self, items, greedy: bool = False):
+    def forward_logits(self, items, greedy: bool = False, want: Optional[dict] = None):
         """Run one step; returns (rows [(seq,row)], logits [R, V] f32 -- or int32 token
-        ids [R] when ``greedy``)."""
+        ids [R] when ``greedy``).  ``want``: see :meth:`prepare`."""
         if not items:
             return [], None
-        si, rows = self.prepare(items, greedy)
+        si, rows = self.prepare(items, greedy, want)
         if si.gather is not None:
             si.prev_bcast = self.prev_sampled_rows
         if self.step_hook is not None:
@@ -520,7 +551,7 @@ class ModelRunner:
         # replay: int32 [ids | pos | slots | ctx | block table | shared_len], then room for
         # the int64 in-flight gather rows (dst, src) and sampled rows of up to B rows
         nb = self.max_blocks
-        n32 = 4 * B + B * nb + 1
+        n32 = 4 * B + B * nb + 1 + (B if self.stateful else 0)
         _, nbytes = _PinnedStager.layout([np.zeros(n32, np.int32)] + [np.zeros(B, np.int64)] * 3)
         raw = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
         i32 = raw[: 4 * n32].view(torch.int32)
@@ -531,12 +562,17 @@ class ModelRunner:
             "slots": i32[2 * B:3 * B].fill_(-1),
             "ctx": i32[3 * B:4 * B].fill_(1),
             "bt": i32[4 * B:4 * B + B * nb].view(B, nb),
-            "shared": i32[4 * B + B * nb:],
+            "shared": i32[4 * B + B * nb:4 * B + B * nb + 1],
         }
+        if self.stateful:  # one sequence per row: its state slot (-1: padding row)
+            st["state_slots"] = i32[4 * B + B * nb + 1:4 * B + B * nb + 1 + B].fill_(-1)
         split, ms = self.decode_split(B)
         st["meta"] = AttnMeta(positions=st["pos"], slots=st["slots"], num_decode=B,
                               block_tables_d=st["bt"], ctx_lens_d=st["ctx"], max_splits=ms,
                               decode_split=split, part_o=po, part_ml=pm)
+        if self.stateful:
+            st["meta"].seq_cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
+            st["meta"].state_slots = st["state_slots"]
         if self.cascade and B >= 2:
             st["shared_len"] = st["shared"]
             self._cascade_meta(st["meta"], B, st["shared_len"])
@@ -578,8 +614,9 @@ class ModelRunner:
         Bg = si.decode_graph
         st = self.graphs.get((Bg, si.greedy)) or self.capture(Bg, si.greedy)
         static = np.concatenate([si.ids, si.positions, si.slots, si.ctx_d, si.tables_d.reshape(-1),
-                                 np.asarray([si.shared_len], dtype=np.int32)]).astype(np.int32, copy=False)
-        if static.size != 4 * Bg + st["bt"].numel() + 1:
+                                 np.asarray([si.shared_len], dtype=np.int32)]
+                                + ([si.state_slots] if self.stateful else [])).astype(np.int32, copy=False)
+        if static.size != 4 * Bg + st["bt"].numel() + 1 + (Bg if self.stateful else 0):
             raise ValueError("decode graph inputs do not match the captured bucket's layout")
         arrays = [static]
         if si.gather is not None:
@@ -621,3 +658,4 @@ class StepInputs:
     gather: Optional[tuple] = None        # (dst rows, src rows): in-flight ids from the previous step
     shared_len: int = 0                   # cascade: leading keys shared by every decode row
     prev_bcast: int = 0                   # TP: rows of driver-sampled previous ids to broadcast
+    state_slots: Optional[np.ndarray] = None  # stateful models: state slot per sequence (prefill seqs, then decode rows)

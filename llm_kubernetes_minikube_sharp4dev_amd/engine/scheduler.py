@@ -37,8 +37,10 @@ class Scheduler:
     def __init__(self, allocator, block_size: int, max_num_seqs: int = 256,
                  max_num_batched_tokens: int = 65536, max_model_len: int = 8192, token_align: int = 256,
                  token_align_wave: int = 0, prefill_hold: int = 0, hold_min_decode: int = 64,
-                 hold_fill: float = 1.0, small_buckets: tuple = (), hold_small: int = 0):
+                 hold_fill: float = 1.0, small_buckets: tuple = (), hold_small: int = 0, state_pool=None):
         self.alloc = allocator
+        # stateful models: a sequence also needs a state slot while it runs (None: stateless model)
+        self.state_pool = state_pool
         # weight-streaming steps (<= small_buckets[-1] rows): prompt prefill is trimmed so the
         # step stays in the row bucket its decode / extend rows already need (the decode GEMMs'
         # cost steps up with the padded row count, 64 / 128 / 192 / 256); the trimmed prompt
@@ -88,6 +90,12 @@ class Scheduler:
 
     # -------------------------------------------------------------- blocks
     def _ensure(self, seq: Sequence, total_tokens: int) -> bool:
+        took_slot = False
+        if self.state_pool is not None and seq.state_slot < 0:
+            if not self.state_pool.num_free:
+                return False
+            seq.state_slot = self.state_pool.acquire()
+            took_slot = True
         need = (total_tokens + self.bs - 1) // self.bs - len(seq.block_table)
         got = []
         try:
@@ -95,6 +103,9 @@ class Scheduler:
                 got.append(self.alloc.allocate())
         except NoFreeBlocks:
             self.alloc.free_all(got)
+            if took_slot:
+                self.state_pool.release(seq.state_slot)
+                seq.state_slot = -1
             return False
         seq.block_table.extend(got)
         return True
@@ -102,6 +113,20 @@ class Scheduler:
     def release(self, seq: Sequence):
         self.alloc.free_all(seq.block_table)
         seq.block_table = []
+        if self.state_pool is not None and seq.state_slot >= 0:
+            self.state_pool.release(seq.state_slot)
+            seq.state_slot = -1
+
+    def admit_forced(self, seq: Sequence, total_tokens: int) -> bool:
+        """Replay mode (LLMEngine.replay_step): make ``seq`` a running sequence, if it is not one yet,
+        and reserve cache blocks (and a state slot) for its first ``total_tokens`` tokens.  No token
+        budget, no preemption: False when the pool cannot hold them."""
+        if not self._ensure(seq, total_tokens):
+            return False
+        if seq.status != Status.RUNNING:
+            seq.status = Status.RUNNING
+            self.running.append(seq)
+        return True
 
     def _preempt(self, seq: Sequence):
         self.release(seq)

@@ -25,6 +25,7 @@ class Sequence:
     req_id: str = field(default_factory=lambda: f"req-{next(_ids)}")
     output_ids: list = field(default_factory=list)
     block_table: list = field(default_factory=list)
+    state_slot: int = -1           # StateSlotPool slot (stateful mixers), -1: none held
     num_computed: int = 0          # tokens whose K/V are in the cache
     num_cached_prefix: int = 0     # tokens served by the prefix cache at admission
     num_hashed_blocks: int = 0     # full blocks already published to the prefix cache

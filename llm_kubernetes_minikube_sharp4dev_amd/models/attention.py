@@ -86,6 +86,13 @@ class AttnMeta:
     # at global position cp_key_start_{p,d}[b] (host ints); queries are replicated
     cp_key_start_p: Optional[list] = None
     cp_key_start_d: Optional[list] = None
+    # stateful mixers (models/ssm.py): every sequence of the step, prefill chunks first and then one
+    # per decode row -- rows [seq_cu[s], seq_cu[s+1]), state slot state_slots[s] (< 0: padding row)
+    seq_cu: Optional[torch.Tensor] = None
+    state_slots: Optional[torch.Tensor] = None
+    max_seq_len: int = 1
+    # sigmoid attention (sigmoid_paged_attention): its 16-query tile list, built once per step
+    sig_tiles: Optional[tuple] = None
 
     @property
     def num_tokens(self) -> int:
@@ -156,6 +163,62 @@ def paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta, Hq: int
         prefill()
     if Bd:
         decode()
+    return out
+
+
+@dataclass
+class SigmoidAttnSpec:
+    """Sigmoid attention: weight = sigmoid(scale q.k - r1_h ln(1 + r2_h (i - j)) + pb_h) over the
+    causal keys, not normalised; q and k unit-RMS per head (no learned weight); no rotation."""
+    heads: int
+    kv_heads: int
+    dim: int           # per-head q / k size
+    vdim: int          # per-head v size
+    scale: float
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "SigmoidAttnSpec":
+        s = cls(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                float(m.get("scale", int(m["dim"]) ** -0.5)))
+        if s.heads % s.kv_heads:
+            raise ValueError(f"heads {s.heads} not a multiple of kv_heads {s.kv_heads}")
+        return s
+
+    @property
+    def qkv_out(self) -> int:
+        return (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
+
+    def cache_shapes(self, num_blocks: int, block_size: int):
+        """K [NB, G, BS, dim] and V key-contiguous [NB, G, vdim, BS] (csrc/attn_sigmoid.hip)."""
+        return ((num_blocks, self.kv_heads, block_size, self.dim), (num_blocks, self.kv_heads, self.vdim, block_size))
+
+    def bytes_per_token(self, dtype) -> int:
+        return self.kv_heads * (self.dim + self.vdim) * torch.tensor([], dtype=dtype).element_size()
+
+
+def sigmoid_paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta, spec: SigmoidAttnSpec, r1, r2, pb,
+                            eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """qkv [T, (H + G) dim + G vdim] straight from the projection: unit-RMS q / k, k / v filed in
+    the paged cache at ``meta.slots``, then prompt rows on the tiled prefill kernel and decode rows
+    on the key-split decode kernel, both reading K / V from the cache (chunked prefill and decode
+    are the same code path as whole prompts).  Returns [T, H vdim]."""
+    H, G, dim, vdim = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    T = qkv.shape[0]
+    if out is None:
+        out = torch.empty(T, H * vdim, dtype=qkv.dtype, device=qkv.device)
+    ops.unitnorm_kv_write(qkv, H, G, dim, vdim, eps, k_cache, v_cache, meta.slots)
+    Tp, Bd = meta.num_prefill_tokens, meta.num_decode
+    if Tp:
+        if meta.sig_tiles is None and qkv.is_cuda:
+            ts, tq = ops.sig_prefill_tiles(meta.q_lens_cpu)
+            meta.sig_tiles = (torch.from_numpy(ts).to(qkv.device, non_blocking=True),
+                              torch.from_numpy(tq).to(qkv.device, non_blocking=True))
+        ops.sigmoid_attention_prefill(qkv[:Tp], k_cache, v_cache, meta.block_tables_p, meta.cu_q, meta.ctx_lens_p,
+                                      H, G, dim, vdim, spec.scale, r1, r2, pb, out[:Tp], tiles=meta.sig_tiles)
+    if Bd:
+        Z = ops.sig_decode_splits(Bd, G, H // G, meta.block_tables_d.shape[1] * k_cache.shape[2])
+        ops.sigmoid_attention_decode(qkv[Tp:Tp + Bd], k_cache, v_cache, meta.block_tables_d, meta.ctx_lens_d, H, G,
+                                     dim, vdim, spec.scale, r1, r2, pb, out[Tp:Tp + Bd], splits=Z)
     return out
 
 

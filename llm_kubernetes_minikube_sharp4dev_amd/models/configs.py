@@ -60,6 +60,98 @@ class EncoderConfig:
         return self.hidden // self.num_heads
 
 
+@dataclass
+class HybridLayer:
+    """One layer of a hybrid decoder: which sequence mixer it has, the mixer's sizes and constants,
+    and its feed-forward (None: the layer has none)."""
+    type: str                    # "attention" (sigmoid attention) | "mamba2"
+    mixer: dict
+    mlp: Optional[dict] = None   # {"kind": "dense", "ff": n}
+
+
+@dataclass
+class LebepelConfig:
+    """The Lebepel design: parallel blocks (one norm feeds the mixer and the feed-forward, their sum
+    scaled by ``residual_mult``) over an f32 residual stream, sigmoid-attention and Mamba-2 mixers
+    in any order, a span of layers run ``loop_times`` times with shared weights (the embedding
+    output added again before each later pass), learned positions, soft-capped logits.
+    Every size and constant comes from the checkpoint's ``config.json`` (:meth:`from_json`)."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layers: list                 # [HybridLayer]
+    max_position: int = 2048
+    norm_eps: float = 1e-5
+    residual_mult: float = 1.0
+    logit_softcap: float = 0.0   # 0: none
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    arch: str = "lebepel"
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    tie_word_embeddings: bool = False
+
+    def layer_runs(self) -> list:
+        """[(layer index, add the embedding output first)] in execution order: the looped span is
+        unrolled; every run has a cache or state of its own."""
+        n = len(self.layers)
+        a, b, t = self.loop_start, self.loop_stop, self.loop_times
+        if not (0 <= a <= b <= n) or t < 1:
+            raise ValueError(f"loop [{a}, {b}) x {t} does not fit {n} layers")
+        runs = [(i, False) for i in range(a)]
+        for k in range(t):
+            runs += [(i, k > 0 and i == a) for i in range(a, b)]
+        return runs + [(i, False) for i in range(b, n)]
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layer_runs())
+
+    @classmethod
+    def from_json(cls, d: dict, name: str = "lebepel") -> "LebepelConfig":
+        layers = [HybridLayer(l["type"], dict(l["mixer"]), dict(l["mlp"]) if l.get("mlp") else None)
+                  for l in d["layers"]]
+        for l in layers:
+            if l.type not in ("attention", "mamba2"):
+                raise ValueError(f"unknown mixer type {l.type!r}")
+            if l.mlp is not None and l.mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"unknown feed-forward kind {l.mlp.get('kind')!r}")
+        loop = d.get("loop") or {}
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=layers,
+                   max_position=int(d["max_positions"]), norm_eps=float((d.get("norm") or {}).get("eps", 1e-5)),
+                   residual_mult=float(d.get("residual_mult", 1.0)), logit_softcap=float(d.get("logit_softcap") or 0.0),
+                   loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+                   loop_times=int(loop.get("times", 1)))
+
+    def to_json(self) -> dict:
+        d = {"architecture": "Lebepel", "vocab": self.vocab_size, "width": self.hidden,
+             "max_positions": self.max_position, "norm": {"eps": self.norm_eps}, "residual_mult": self.residual_mult,
+             "logit_softcap": self.logit_softcap,
+             "layers": [{"type": l.type, "mixer": dict(l.mixer), "mlp": dict(l.mlp) if l.mlp else None}
+                        for l in self.layers]}
+        if self.loop_times > 1 or self.loop_stop > self.loop_start:
+            d["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        return d
+
+
+def lebepel_layers(n: int, hidden: int, heads: int, kv_heads: int, head_dim: int, ff: int, ssm_heads: int, ssm_p: int,
+                   ssm_state: int, ssm_groups: int = 1, conv: int = 4, norm_groups: int = 1, pattern=("attention", "mamba2"),
+                   scale: Optional[float] = None) -> list:
+    """``n`` layers cycling through ``pattern`` with one set of mixer sizes (presets and benchmarks)."""
+    out = []
+    for i in range(n):
+        t = pattern[i % len(pattern)]
+        if t == "attention":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim,
+                     "scale": scale if scale is not None else head_dim ** -0.5}
+        else:
+            mixer = {"heads": ssm_heads, "vdim": ssm_p, "state": ssm_state, "groups": ssm_groups, "conv": conv,
+                     "norm_groups": norm_groups}
+        out.append(HybridLayer(t, mixer, {"kind": "dense", "ff": ff} if ff else None))
+    return out
+
+
 LLAMA3_SCALING = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                   "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
 
@@ -82,6 +174,16 @@ DECODERS = {
                               bos_token_id=2, eos_token_ids=(2,)),
 }
 
+DECODERS.update({
+    # hybrid sigmoid-attention / Mamba-2 decoders (random-init presets; checkpoints bring their own config.json)
+    "lebepel-tiny": LebepelConfig("lebepel-tiny", 32768, 128, lebepel_layers(3, 128, 4, 2, 32, 256, 4, 16, 16, 2, 4, 2,
+                                                                              ("mamba2", "attention", "mamba2")),
+                                  max_position=1024, residual_mult=0.7, logit_softcap=20.0, loop_start=1, loop_stop=3,
+                                  loop_times=2),
+    "lebepel-1b": LebepelConfig("lebepel-1b", 32768, 2048, lebepel_layers(16, 2048, 16, 4, 128, 5632, 64, 64, 128, 8, 4, 8),
+                                max_position=8192, residual_mult=1.0, logit_softcap=30.0),
+})
+
 ENCODERS = {
     "bge-base": EncoderConfig("bge-base", "bert", 12, 768, 12, 3072, 30522, pooling="cls"),
     "minilm-l6": EncoderConfig("minilm-l6", "bert", 6, 384, 12, 1536, 30522, pooling="mean"),
@@ -94,7 +196,7 @@ ENCODERS = {
 }
 
 
-def decoder_config(name: str, **overrides) -> DecoderConfig:
+def decoder_config(name: str, **overrides):
     cfg = dataclasses.replace(DECODERS[name])
     for k, v in overrides.items():
         setattr(cfg, k, v)
@@ -108,7 +210,19 @@ def encoder_config(name: str, **overrides) -> EncoderConfig:
     return cfg
 
 
-def param_count(cfg: DecoderConfig) -> int:
+def param_count(cfg) -> int:
+    if isinstance(cfg, LebepelConfig):
+        W, n = cfg.hidden, (cfg.vocab_size * 2 + cfg.max_position + 1) * cfg.hidden
+        for l in cfg.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (m["heads"] + m["kv_heads"]) * m["dim"] + 2 * W * m["kv_heads"] * m["vdim"] \
+                    + W * (m["heads"] - m["kv_heads"]) * m["vdim"]
+            else:
+                inner = m["heads"] * m["vdim"]
+                n += W * (2 * inner + 2 * m["groups"] * m["state"] + m["heads"]) + W * inner
+            n += W + (3 * W * l.mlp["ff"] if l.mlp else 0)
+        return n
     H, I, L, V = cfg.hidden, cfg.intermediate, cfg.num_layers, cfg.vocab_size
     qkv = H * (cfg.num_heads + 2 * cfg.num_kv_heads) * cfg.head_dim
     o = cfg.num_heads * cfg.head_dim * H

@@ -15,6 +15,9 @@ import torch
 
 from . import reference as ref
 from ._ext import available, force_reference, lib, use_hip  # noqa: F401
+from .mixers import (conv_silu, embed_pos, gated_group_rmsnorm, linear_swiglu_any, sig_decode_splits,  # noqa: F401
+                     sig_prefill_tiles, sigattn_supported, sigmoid_attention_decode, sigmoid_attention_prefill,
+                     softcap, ssm_scan, stream_rmsnorm, unitnorm_kv_write)
 
 __all__ = [
     "rmsnorm", "layernorm", "embed_layernorm", "silu_mul", "gelu_", "relu_", "rope_kv_",

@@ -1,0 +1,262 @@
+"""Entry points of the sequence-mixer kernels beside softmax attention: an f32 residual stream
+(``csrc/stream_f32.hip``), sigmoid attention with a log-distance penalty over a paged cache
+(``csrc/attn_sigmoid.hip``) and a Mamba-2 style state-space mixer (``csrc/ssm.hip``).
+
+GPU tensors go to the HIP kernels (bf16 or f32 activations); CPU tensors to the torch
+implementations below, which keep the kernels' layouts and their split of what is 32-bit:
+
+* K cache ``[blocks, G, BS, dim]``, V cache key-contiguous ``[blocks, G, vdim, BS]``;
+* sequences of a step: rows ``[cu[s], cu[s+1])``, state slot ``slots[s]`` (< 0: padding row),
+  fresh state when ``positions[cu[s]] == 0``;
+* conv state ``[slots, taps - 1, C]`` (activation dtype), SSM state ``[slots, heads, P, N]`` f32.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from ._ext import lib, use_hip
+
+__all__ = ["embed_pos", "stream_rmsnorm", "softcap", "linear_swiglu_any", "unitnorm_kv_write", "sig_prefill_tiles", "sig_decode_splits",
+           "sigmoid_attention_prefill", "sigmoid_attention_decode", "sigattn_supported", "conv_silu", "ssm_scan",
+           "gated_group_rmsnorm"]
+
+SIG_TILE_ROWS = 16       # queries per wave of the prefill kernel
+SIG_MAX_HEAD = 256       # largest per-head q/k or v size the kernels are built for
+
+
+# ------------------------------------------------------------------ f32 residual stream
+def embed_pos(ids, positions, tok, pos, keep_copy: bool = False):
+    """x f32 [T, W] = tok[ids] + pos[positions]; with ``keep_copy`` a second tensor of the same
+    values (for models that add the embedding output to the stream again)."""
+    if use_hip(tok):
+        r = lib().embed_pos(ids, positions, tok, pos, keep_copy)
+        return (r[0], r[1]) if keep_copy else (r[0], None)
+    x = tok[ids.long()].float() + pos[positions.long()].float()
+    return x, (x.clone() if keep_copy else None)
+
+
+def stream_rmsnorm(x, a=None, b=None, e=None, mult: float = 1.0, w=None, w_offset: float = 0.0, eps: float = 1e-5,
+                   idx=None, out_dtype=torch.bfloat16):
+    """``x += mult * (a + b) + e`` in place (f32), then ``x / sqrt(mean(x^2) + eps) * (w_offset + w)``
+    in ``out_dtype``.  With ``idx`` (int64 rows) only those rows are computed and ``x`` is left
+    as it was."""
+    if use_hip(x):
+        return lib().stream_rmsnorm(x, a, b, e, float(mult), w, float(w_offset), float(eps), idx, out_dtype)
+    v = x if idx is None else x.index_select(0, idx)
+    sel = (lambda t: t) if idx is None else (lambda t: t.index_select(0, idx))
+    d = None
+    for t in (a, b):
+        if t is not None:
+            d = sel(t).float() if d is None else d + sel(t).float()
+    if d is not None:
+        v = v + mult * d
+    if e is not None:
+        v = v + sel(e)
+    if idx is None and v is not x:
+        x.copy_(v)
+    h = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        h = h * (w_offset + w.float())
+    return h.to(out_dtype)
+
+
+def softcap(z, cap: float):
+    """``cap * tanh(z / cap)`` as f32 (cap <= 0: a plain f32 copy)."""
+    if use_hip(z):
+        return lib().softcap(z, float(cap))
+    zf = z.float()
+    return cap * torch.tanh(zf / cap) if cap > 0 else zf
+
+
+def linear_swiglu_any(x, w_gate_up):
+    """silu(x Wg^T) * (x Wu^T) for a fused [Wg; Wu] weight in bf16 (the GEMM's SwiGLU epilogue) or,
+    for f32 activations on the GPU, a true-f32 library product and an f32 activation kernel."""
+    from . import linear_swiglu
+
+    if use_hip(x) and x.dtype == torch.float32:
+        return lib().silu_mul_f32(F.linear(x, w_gate_up))
+    return linear_swiglu(x, w_gate_up)
+
+
+# ------------------------------------------------------------------ sigmoid attention
+def sigattn_supported(H: int, G: int, dim: int, vdim: int, block_size: int, dtype) -> bool:
+    ev = 16 // torch.tensor([], dtype=dtype).element_size()
+    return (H % G == 0 and dim % ev == 0 and vdim % ev == 0 and block_size % 16 == 0
+            and max(dim, vdim) <= SIG_MAX_HEAD)
+
+
+def unitnorm_kv_write(qkv, H: int, G: int, dim: int, vdim: int, eps: float, k_cache, v_cache, slots):
+    """Rows ``[q: H dim | k: G dim | v: G vdim]``: q and k become x / sqrt(mean(x^2) + eps) per head
+    (f32 arithmetic; q in place, k into the cache), v goes into the cache.  Slots < 0 cache nothing."""
+    if use_hip(qkv):
+        lib().unitnorm_kv_write(qkv, H, G, dim, vdim, float(eps), k_cache, v_cache, slots)
+        return qkv
+    T = qkv.shape[0]
+    qk = qkv[:, : (H + G) * dim].float().view(T, H + G, dim)
+    qk = qk / torch.sqrt(qk.pow(2).mean(-1, keepdim=True) + eps)
+    qkv[:, : (H + G) * dim] = qk.reshape(T, -1).to(qkv.dtype)
+    BS = k_cache.shape[2]
+    sl = slots[:T].long()
+    ok = sl >= 0
+    blk, off = sl[ok] // BS, sl[ok] % BS
+    k_cache[blk, :, off, :] = qkv[ok, H * dim:(H + G) * dim].view(-1, G, dim)
+    v_cache[blk, :, :, off] = qkv[ok, (H + G) * dim:].view(-1, G, vdim)
+    return qkv
+
+
+def sig_prefill_tiles(q_lens: Sequence[int]):
+    """(tile_seq, tile_q0) int32: one entry per 16-query tile of each chunk; a tile's cost grows with
+    its position in the sequence, so the later tiles of a chunk are listed (and start) first."""
+    seq, q0 = [], []
+    for b, n in enumerate(q_lens):
+        for s in range(((n + SIG_TILE_ROWS - 1) // SIG_TILE_ROWS - 1) * SIG_TILE_ROWS, -1, -SIG_TILE_ROWS):
+            seq.append(b)
+            q0.append(s)
+    return np.asarray(seq, dtype=np.int32), np.asarray(q0, dtype=np.int32)
+
+
+def sig_decode_splits(B: int, G: int, rep: int, max_context: int) -> int:
+    """Workgroups per (sequence, kv group) of the decode kernel: enough to give the chip about two
+    workgroups per CU, never more than one per 128 keys (a workgroup's 4 waves take 32 keys each
+    per round).  Static per (batch bucket, model, max context): safe to capture."""
+    groups = max(1, B * G * ((rep + 15) // 16))
+    return int(max(1, min(512 // groups, (max_context + 127) // 128)))
+
+
+def _gather_kv(k_cache, v_cache, table, n):
+    BS = k_cache.shape[2]
+    nb = (n + BS - 1) // BS
+    bt = table[:nb].long()
+    k = k_cache[bt].permute(0, 2, 1, 3).reshape(nb * BS, k_cache.shape[1], -1)[:n]     # [n, G, dim]
+    v = v_cache[bt].permute(0, 3, 1, 2).reshape(nb * BS, v_cache.shape[1], -1)[:n]     # [n, G, vdim]
+    return k.float(), v.float()
+
+
+def _sig_rows(q, k, v, qpos, scale, r1, r2, pb):
+    """q f32 [S, H, dim] at positions qpos [S]; k/v f32 [n, G, *] at positions 0..n-1."""
+    H, G = q.shape[1], k.shape[1]
+    rep = H // G
+    kk = k.repeat_interleave(rep, dim=1)
+    vv = v.repeat_interleave(rep, dim=1)
+    s = torch.einsum("ihd,jhd->hij", q, kk) * scale
+    d = qpos.view(-1, 1) - torch.arange(k.shape[0], device=q.device).view(1, -1)
+    pen = r1.view(-1, 1, 1) * torch.log(1.0 + r2.view(-1, 1, 1) * d.clamp(min=0).float()[None])
+    wgt = torch.sigmoid(s - pen + pb.view(-1, 1, 1)) * (d >= 0)[None]
+    return torch.einsum("hij,jhd->ihd", wgt, vv)
+
+
+def sigmoid_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H: int, G: int, dim: int, vdim: int,
+                              scale: float, r1, r2, pb, out, tiles=None, q_lens_cpu=None):
+    """Causal sigmoid attention of query chunks over their sequences' cached keys (the chunk's own
+    keys included).  q: rows whose first H * dim columns are the unit-RMS queries; out [T, H * vdim]."""
+    if use_hip(q):
+        if tiles is None:
+            ql = q_lens_cpu if q_lens_cpu is not None else (cu_q[1:] - cu_q[:-1]).tolist()
+            ts, tq = sig_prefill_tiles(ql)
+            tiles = (torch.from_numpy(ts).to(q.device), torch.from_numpy(tq).to(q.device))
+        lib().sigattn_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, tiles[0], tiles[1], H, G, dim, vdim,
+                              float(scale), r1, r2, pb, out)
+        return out
+    cu = cu_q.tolist()
+    for b in range(len(cu) - 1):
+        s0, s1 = cu[b], cu[b + 1]
+        n = int(ctx_lens[b])
+        k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
+        qq = q[s0:s1, : H * dim].float().view(s1 - s0, H, dim)
+        qpos = torch.arange(n - (s1 - s0), n, device=q.device)
+        out[s0:s1, : H * vdim] = _sig_rows(qq, k, v, qpos, scale, r1, r2, pb).reshape(s1 - s0, H * vdim).to(out.dtype)
+    return out
+
+
+def sigmoid_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, H: int, G: int, dim: int, vdim: int,
+                             scale: float, r1, r2, pb, out, splits: int = 1, part=None):
+    """One query row per sequence at its last position (ctx - 1) over all its cached keys."""
+    B = q.shape[0]
+    if use_hip(q):
+        if splits > 1 and part is None:
+            part = torch.empty(B * H * splits * vdim, dtype=torch.float32, device=q.device)
+        lib().sigattn_decode(q, k_cache, v_cache, block_tables, ctx_lens, int(splits), H, G, dim, vdim, float(scale),
+                             r1, r2, pb, out, part)
+        return out
+    for b in range(B):
+        n = int(ctx_lens[b])
+        k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
+        qq = q[b:b + 1, : H * dim].float().view(1, H, dim)
+        qpos = torch.tensor([n - 1], device=q.device)
+        out[b:b + 1, : H * vdim] = _sig_rows(qq, k, v, qpos, scale, r1, r2, pb).reshape(1, H * vdim).to(out.dtype)
+    return out
+
+
+# ------------------------------------------------------------------ state-space mixer
+def conv_silu(u, col0: int, C: int, w, bias, state, cu, slots, positions, max_len: int):
+    """silu(causal depthwise conv + bias) of columns [col0, col0 + C) of ``u``, per sequence, reading
+    the inputs before a chunk from ``state`` and leaving the sequence's last ``taps - 1`` inputs there.
+    w f32 [C, taps] (last column = the current token), bias f32 [C] or None."""
+    if use_hip(u):
+        return lib().conv_silu(u, col0, C, w, bias, state, cu, slots, positions, int(max_len))
+    taps = w.shape[1]
+    out = torch.zeros(u.shape[0], C, dtype=u.dtype, device=u.device)
+    cul, sl = cu.tolist(), slots.tolist()
+    for s in range(len(cul) - 1):
+        r0, r1 = cul[s], cul[s + 1]
+        if sl[s] < 0 or r1 <= r0:
+            continue
+        x = u[r0:r1, col0:col0 + C]
+        if taps > 1:
+            prev = state[sl[s]] if int(positions[r0]) > 0 else torch.zeros_like(state[sl[s]])
+            full = torch.cat([prev, x], 0)                                    # [taps - 1 + n, C]
+            state[sl[s]] = full[-(taps - 1):]
+        else:
+            full = x
+        ff = full.float()
+        acc = torch.zeros(r1 - r0, C, dtype=torch.float32, device=u.device)
+        for k in range(taps):
+            acc += ff[k:k + r1 - r0] * w[:, k]
+        if bias is not None:
+            acc += bias
+        out[r0:r1] = F.silu(acc).to(u.dtype)
+    return out
+
+
+def ssm_scan(xbc, dt, heads: int, P: int, N: int, groups: int, dt_bias, A_log, D, state, cu, slots, positions):
+    """y f32 [T, heads * P]: per head, S_t = exp(-exp(A_log) dt_t) S_{t-1} + dt_t B_t x_t^T and
+    y_t = S_t^T C_t + D x_t with dt_t = softplus(dt_t + dt_bias); x | B | C are the columns of
+    ``xbc``; the f32 state of each sequence is read from / left in ``state[slot]`` ([heads, P, N])."""
+    if use_hip(xbc):
+        return lib().ssm_scan(xbc, dt, heads, P, N, groups, dt_bias, A_log, D, state, cu, slots, positions)
+    inner = heads * P
+    y = torch.zeros(xbc.shape[0], inner, dtype=torch.float32, device=xbc.device)
+    cul, sl = cu.tolist(), slots.tolist()
+    nA = -torch.exp(A_log.float())
+    hg = heads // groups
+    for s in range(len(cul) - 1):
+        r0, r1 = cul[s], cul[s + 1]
+        if sl[s] < 0 or r1 <= r0:
+            continue
+        S = state[sl[s]].clone() if int(positions[r0]) > 0 else torch.zeros_like(state[sl[s]])   # [heads, P, N]
+        rows = xbc[r0:r1].float()
+        x = rows[:, :inner].view(-1, heads, P)
+        Bm = rows[:, inner:inner + groups * N].view(-1, groups, N).repeat_interleave(hg, dim=1)
+        Cm = rows[:, inner + groups * N:].view(-1, groups, N).repeat_interleave(hg, dim=1)
+        dts = F.softplus(dt[r0:r1].float() + dt_bias, threshold=20.0)
+        dA = torch.exp(nA * dts)
+        for t in range(r1 - r0):
+            S = dA[t].view(-1, 1, 1) * S + (dts[t].view(-1, 1) * x[t]).unsqueeze(-1) * Bm[t].unsqueeze(1)
+            y[r0 + t] = (torch.einsum("hpn,hn->hp", S, Cm[t]) + D.view(-1, 1) * x[t]).reshape(-1)
+        state[sl[s]] = S
+    return y
+
+
+def gated_group_rmsnorm(y, z, w, ngroups: int, eps: float):
+    """(y * silu(z)) normalised to unit RMS within each of ``ngroups`` equal column groups, times w;
+    y f32, z and the result in the activation dtype."""
+    if use_hip(y):
+        return lib().gated_group_rmsnorm(y, z, w, int(ngroups), float(eps))
+    T, inner = y.shape
+    v = (y * F.silu(z.float())).view(T, ngroups, inner // ngroups)
+    v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    return (v.reshape(T, inner) * w).to(z.dtype)

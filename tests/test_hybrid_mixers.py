@@ -1,0 +1,331 @@
+"""The hybrid decoder's mechanisms, each alone, against the plain float64 implementations of
+``hybrid_oracle``: the framework's ops over a paged cache / state slots, whole sequences and cut
+into portions, on the CPU path and (``gpu`` marker) on the HIP kernels in f32 and bf16."""
+import math
+
+import pytest
+import torch
+
+import hybrid_oracle as O
+from llm_kubernetes_minikube_sharp4dev_amd import ops
+from llm_kubernetes_minikube_sharp4dev_amd.models.attention import AttnMeta, SigmoidAttnSpec, sigmoid_paged_attention
+from llm_kubernetes_minikube_sharp4dev_amd.models.ssm import Mamba2Spec, mamba2_mixer
+
+CPU32 = pytest.param("cpu", torch.float32, id="cpu-f32")
+GPU32 = pytest.param("cuda", torch.float32, id="gpu-f32", marks=pytest.mark.gpu)
+GPU16 = pytest.param("cuda", torch.bfloat16, id="gpu-bf16", marks=pytest.mark.gpu)
+ALL = [CPU32, GPU32, GPU16]
+
+
+def tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 3e-2
+
+
+def rel_err(got, want):
+    want = want.double()
+    return float((got.double().cpu() - want).abs().max() / want.abs().max().clamp_min(1e-9))
+
+
+def rnd(g, *shape, scale=1.0):
+    return torch.randn(*shape, generator=g, dtype=torch.float64) * scale
+
+
+def q16(t):
+    """Values a bf16 tensor holds exactly, so both sides of a comparison start from the same weights."""
+    return t.to(torch.bfloat16).to(torch.float64)
+
+
+# ---------------------------------------------------------------------------- residual stream
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_embed_stream_norm_softcap(device, dtype):
+    g = torch.Generator().manual_seed(1)
+    V, P, W, T = 50, 40, 72, 9
+    tok, pos = q16(rnd(g, V, W)), q16(rnd(g, P, W))
+    ids = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    ps = torch.randint(0, P, (T,), generator=g, dtype=torch.int32)
+    x, e = ops.embed_pos(ids.to(device), ps.to(device), tok.to(dtype).to(device), pos.to(dtype).to(device), keep_copy=True)
+    want = tok[ids.long()] + pos[ps.long()]
+    assert x.dtype == torch.float32 and rel_err(x, want) < 1e-6 and torch.equal(x, e) and x.data_ptr() != e.data_ptr()
+    a, b, w = q16(rnd(g, T, W)), q16(rnd(g, T, W)), q16(rnd(g, W, scale=0.1))
+    eps, m = 1e-3, 0.37
+    xs = want + m * (a + b) + want
+    hw = O.offset_rmsnorm(xs, w, eps)
+    x0 = x.clone()
+    h = ops.stream_rmsnorm(x, a.to(dtype).to(device), b.to(dtype).to(device), e, m, w.float().to(device), 1.0, eps,
+                           out_dtype=dtype)
+    assert rel_err(x, xs) < 1e-6 and rel_err(h, hw) < tol(dtype) / 4
+    # one input only, no weight offset, rows picked by index: the stream is left alone
+    idx = torch.tensor([7, 0, 3], device=device)
+    x1 = x0.clone()
+    h2 = ops.stream_rmsnorm(x1, a.to(dtype).to(device), None, None, m, w.float().to(device), 0.0, eps, idx=idx, out_dtype=dtype)
+    assert torch.equal(x1, x0)
+    assert rel_err(h2, (O.unit_rms(want + m * a, eps) * w)[idx.cpu()]) < tol(dtype) / 4
+    z = q16(rnd(g, 4, 300, scale=25.0))
+    c = ops.softcap(z.to(dtype).to(device), 11.0)
+    assert c.dtype == torch.float32 and rel_err(c, 11.0 * torch.tanh(z / 11.0)) < 1e-5
+    assert rel_err(ops.softcap(z.to(dtype).to(device), 0.0), z) < 1e-6
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_swiglu_any_dtype(device, dtype):
+    g = torch.Generator().manual_seed(2)
+    h, wgu = q16(rnd(g, 5, 64)), q16(rnd(g, 2 * 48, 64, scale=0.2))
+    got = ops.linear_swiglu_any(h.to(dtype).to(device), wgu.to(dtype).to(device))
+    gt = h @ wgu[:48].T
+    assert rel_err(got, gt * torch.sigmoid(gt) * (h @ wgu[48:].T)) < tol(dtype)
+
+
+# ---------------------------------------------------------------------------- sigmoid attention
+class PagedSeqs:
+    """A paged cache with shuffled blocks and block tables for a few sequences."""
+
+    def __init__(self, spec, lens, bs, device, dtype, seed=0):
+        g = torch.Generator().manual_seed(seed)
+        nb = [-(-n // bs) for n in lens]
+        perm = torch.randperm(sum(nb) + 3, generator=g).tolist()
+        self.tables, k = [], 0
+        for n in nb:
+            self.tables.append(perm[k:k + n])
+            k += n
+        ks, vs = spec.cache_shapes(sum(nb) + 3, bs)
+        self.kc = torch.zeros(ks, dtype=dtype, device=device)
+        self.vc = torch.zeros(vs, dtype=dtype, device=device)
+        self.bs, self.device = bs, device
+
+    def meta(self, chunks=(), decodes=()):
+        """chunks: [(seq, start, n)] prompt portions; decodes: [(seq, pos)] single tokens."""
+        width = max(len(t) for t in self.tables)
+        pos, slots = [], []
+        for s, st, n in list(chunks) + [(s, p, 1) for s, p in decodes]:
+            for i in range(st, st + n):
+                pos.append(i)
+                slots.append(self.tables[s][i // self.bs] * self.bs + i % self.bs)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=self.device)
+        bt = lambda ss: i32([self.tables[s] + [0] * (width - len(self.tables[s])) for s in ss])
+        m = AttnMeta(positions=i32(pos), slots=i32(slots), num_prefill_tokens=sum(n for _, _, n in chunks),
+                     num_prefill_seqs=len(chunks), num_decode=len(decodes))
+        if chunks:
+            cu = [0]
+            for _, _, n in chunks:
+                cu.append(cu[-1] + n)
+            m.cu_q, m.ctx_lens_p, m.block_tables_p = i32(cu), i32([st + n for _, st, n in chunks]), bt([s for s, _, _ in chunks])
+            m.q_lens_cpu, m.ctx_lens_cpu = [n for _, _, n in chunks], [st + n for _, st, n in chunks]
+        if decodes:
+            m.block_tables_d, m.ctx_lens_d = bt([s for s, _ in decodes]), i32([p + 1 for _, p in decodes])
+        lens = [n for _, _, n in chunks] + [1] * len(decodes)
+        cu = [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
+        m.seq_cu, m.max_seq_len = i32(cu), max(lens)
+        return m
+
+
+def attn_weights(g, spec, W):
+    d = dict(wq=rnd(g, spec.heads * spec.dim, W, scale=W ** -0.5), bq=rnd(g, spec.heads * spec.dim, scale=0.1),
+             wk=rnd(g, spec.kv_heads * spec.dim, W, scale=W ** -0.5), bk=rnd(g, spec.kv_heads * spec.dim, scale=0.1),
+             wv=rnd(g, spec.kv_heads * spec.vdim, W, scale=W ** -0.5), bv=rnd(g, spec.kv_heads * spec.vdim, scale=0.1),
+             wo=rnd(g, W, spec.heads * spec.vdim, scale=(spec.heads * spec.vdim) ** -0.5), bo=rnd(g, W, scale=0.1),
+             r1=rnd(g, spec.heads, scale=0.2) + 0.6, r2=torch.rand(spec.heads, generator=g, dtype=torch.float64) + 0.1,
+             pb=rnd(g, spec.heads, scale=0.5))
+    return {k: q16(v) for k, v in d.items()}
+
+
+def run_attention(spec, w, hs, schedule, bs, device, dtype, eps=1e-5):
+    """hs: per-sequence inputs [T_s, W]; schedule: steps of ([(seq, start, n)], [(seq, pos)]).
+    Returns per-sequence outputs of the framework path (projections included)."""
+    cache = PagedSeqs(spec, [h.shape[0] for h in hs], bs, device, dtype)
+    dev = lambda t, dt=dtype: t.to(dt).to(device)
+    wqkv, bqkv = dev(torch.cat([w["wq"], w["wk"], w["wv"]])), dev(torch.cat([w["bq"], w["bk"], w["bv"]]))
+    wo, bo = dev(w["wo"]), dev(w["bo"])
+    r1, r2, pb = (dev(w[k], torch.float32) for k in ("r1", "r2", "pb"))
+    outs = [torch.zeros(h.shape[0], w["wo"].shape[0], dtype=torch.float64) for h in hs]
+    for chunks, decodes in schedule:
+        meta = cache.meta(chunks, decodes)
+        rows = [hs[s][st:st + n] for s, st, n in chunks] + [hs[s][p:p + 1] for s, p in decodes]
+        qkv = ops.linear(dev(torch.cat(rows)), wqkv, bqkv)
+        att = sigmoid_paged_attention(qkv, cache.kc, cache.vc, meta, spec, r1, r2, pb, eps)
+        y = ops.linear(att, wo, bo).double().cpu()
+        r = 0
+        for s, st, n in list(chunks) + [(s, p, 1) for s, p in decodes]:
+            outs[s][st:st + n] = y[r:r + n]
+            r += n
+    return outs
+
+
+def oracle_attention(spec, w, h, fast=True, eps=1e-5):
+    f = O.sigmoid_attention_fast if fast else O.sigmoid_attention
+    return f(h, w["wq"], w["bq"], w["wk"], w["bk"], w["wv"], w["bv"], w["wo"], w["bo"], w["r1"], w["r2"], w["pb"],
+             spec.heads, spec.kv_heads, spec.dim, spec.vdim, spec.scale, eps)
+
+
+def test_oracle_forms_agree():
+    g = torch.Generator().manual_seed(3)
+    spec = SigmoidAttnSpec(4, 2, 8, 16, 0.3)
+    w, h = attn_weights(g, spec, 24), rnd(g, 11, 24)
+    assert rel_err(oracle_attention(spec, w, h, True), oracle_attention(spec, w, h, False)) < 1e-12
+
+
+SPECS = [SigmoidAttnSpec(4, 4, 32, 32, 0.2), SigmoidAttnSpec(6, 2, 48, 16, 0.15), SigmoidAttnSpec(8, 1, 16, 64, 0.25),
+         SigmoidAttnSpec(2, 1, 80, 40, 0.11), SigmoidAttnSpec(20, 1, 8, 8, 0.4), SigmoidAttnSpec(2, 2, 136, 200, 0.09)]
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("spec", SPECS, ids=lambda s: f"h{s.heads}g{s.kv_heads}d{s.dim}v{s.vdim}")
+def test_sigmoid_attention_whole_chunked_decoded(spec, device, dtype):
+    """Whole prompts, portions cut at and off page borders (down to two tokens, one token first),
+    and token-by-token decoding give the same rows; two sequences share every step."""
+    g = torch.Generator().manual_seed(4)
+    W, bs = 48, 16
+    w = attn_weights(g, spec, W)
+    hs = [q16(rnd(g, 70, W)), q16(rnd(g, 37, W))]
+    want = [oracle_attention(spec, w, h) for h in hs]
+    whole = run_attention(spec, w, hs, [([(0, 0, 70), (1, 0, 37)], [])], bs, device, dtype)
+    sched = [([(0, 0, 1), (1, 0, 17)], []), ([(0, 1, 2), (1, 17, 15)], []), ([(0, 3, 29)], [(1, 32)]),
+             ([(0, 32, 2)], [(1, 33)]), ([(0, 34, 30)], [(1, 34)]), ([], [(0, 64), (1, 35)]), ([(0, 65, 3)], [(1, 36)]),
+             ([], [(0, 68)]), ([], [(0, 69)])]
+    cut = run_attention(spec, w, hs, sched, bs, device, dtype)
+    for s in range(2):
+        assert rel_err(whole[s], want[s]) < tol(dtype)
+        assert rel_err(cut[s], want[s]) < tol(dtype)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_sigmoid_attention_one_far_key_stands_out(device, dtype):
+    """Every weight is pushed to ~0 by a large negative head bias except where one query and one
+    key are aligned and scaled up: the output row must be that key's value, through a context of
+    hundreds of keys and several pages, in a prompt portion and in a decode row; moving the key
+   , and a query that sits BEFORE the key sees nothing."""
+    spec = SigmoidAttnSpec(2, 1, 16, 16, 1.0)
+    T, bs, far = 300, 16, 5
+    cache = PagedSeqs(spec, [T], bs, device, dtype)
+    g = torch.Generator().manual_seed(5)
+    k = rnd(g, T, 16, scale=0.05)
+    v = q16(rnd(g, T, 16))
+    q = rnd(g, T, 2, 16, scale=0.05)
+    key_dir = torch.zeros(16, dtype=torch.float64)
+    key_dir[3] = 4.0            # unit RMS after the norm: sqrt(16) on one axis
+    k[:, 3] = 0.0               # every other key is orthogonal to the aligned queries: their score is 0
+    k[far] = key_dir
+    for row in (far - 1, 250, T - 1):
+        q[row, :] = key_dir
+    r1 = torch.tensor([0.0, 0.5]); r2 = torch.tensor([1.0, 2.0]); pb = torch.tensor([-12.0, -12.0])
+    scale = 1.25                 # aligned unit-RMS vectors: q.k = 16 -> score 20
+    spec = SigmoidAttnSpec(2, 1, 16, 16, scale)
+    rows = torch.cat([q.reshape(T, 32), k, v], 1).to(dtype).to(device)
+    f32 = lambda t: t.float().to(device)
+    m = cache.meta([(0, 0, T - 1)], [])
+    out = sigmoid_paged_attention(rows[:T - 1].clone(), cache.kc, cache.vc, m, spec, f32(r1), f32(r2), f32(pb), 1e-6)
+    m = cache.meta([], [(0, T - 1)])
+    dec = sigmoid_paged_attention(rows[T - 1:].clone(), cache.kc, cache.vc, m, spec, f32(r1), f32(r2), f32(pb), 1e-6)
+    out = torch.cat([out, dec]).double().cpu().view(T, 2, 16)
+    for row in (250, T - 1):
+        for hd in range(2):
+            pen = float(r1[hd]) * math.log(1.0 + float(r2[hd]) * (row - far))
+            wgt = 1.0 / (1.0 + math.exp(-(20.0 - pen - 12.0)))
+            assert wgt > 0.99
+            assert (out[row, hd] - wgt * v[far]).abs().max() < 0.15, (row, hd)
+    assert out[far - 1].abs().max() < 0.05      # the key lies in that query's future
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_distance_penalty_and_bias_per_head(device, dtype):
+    """Zero q / k: every score is exactly -r1 ln(1 + r2 d) + pb, so with v = one-hot(position) the
+    output spells out the weight of every distance, per head (heads with different constants,
+    sharing one kv head)."""
+    T, bs = 45, 16
+    spec = SigmoidAttnSpec(3, 1, 8, 48, 0.7)
+    cache = PagedSeqs(spec, [T], bs, device, dtype)
+    v = torch.eye(T, 48, dtype=torch.float64)
+    rows = torch.cat([torch.zeros(T, 3 * 8 + 8, dtype=torch.float64), v], 1).to(dtype).to(device)
+    r1 = torch.tensor([0.9, 0.0, 2.0]); r2 = torch.tensor([0.5, 3.0, 0.05]); pb = torch.tensor([0.3, -1.0, 1.5])
+    f32 = lambda t: t.float().to(device)
+    m = cache.meta([(0, 0, T)], [])
+    out = sigmoid_paged_attention(rows, cache.kc, cache.vc, m, spec, f32(r1), f32(r2), f32(pb), 1e-6)
+    out = out.double().cpu().view(T, 3, 48)
+    for hd in range(3):
+        for i in (0, 1, 15, 16, 17, 31, 32, 44):
+            d = i - torch.arange(T, dtype=torch.float64)
+            want = torch.where(d >= 0, torch.sigmoid(-r1[hd].double() * torch.log(1 + r2[hd].double() * d.clamp(min=0)) + pb[hd]),
+                               torch.zeros_like(d))
+            assert (out[i, hd, :T] - want).abs().max() < (1e-5 if dtype == torch.float32 else 4e-3), (hd, i)
+
+
+# ---------------------------------------------------------------------------- state-space mixer
+def mamba_weights(g, spec, W):
+    d = dict(w_in=rnd(g, spec.proj_out, W, scale=W ** -0.5), conv_w=rnd(g, spec.conv_channels, spec.conv, scale=0.4),
+             conv_b=rnd(g, spec.conv_channels, scale=0.1), dt_bias=rnd(g, spec.heads, scale=0.5) - 0.5,
+             a_log=rnd(g, spec.heads, scale=0.4) - 0.5, d_skip=rnd(g, spec.heads, scale=0.3) + 1.0,
+             norm_w=rnd(g, spec.inner, scale=0.2) + 1.0, w_out=rnd(g, W, spec.inner, scale=spec.inner ** -0.5))
+    return {k: q16(v) for k, v in d.items()}
+
+
+def run_mamba(spec, w, hs, schedule, slots, device, dtype, eps=1e-5, nslots=4, poison=True):
+    """schedule: steps of [(seq, start, n)]; slots: state slot of each sequence."""
+    conv, ssm = spec.make_state(nslots, dtype, device)
+    if poison:  # whatever an earlier owner left in a slot must not matter
+        conv.fill_(3.0)
+        ssm.fill_(-2.0)
+    dev = lambda t, dt=dtype: t.to(dt).to(device)
+    f32 = lambda t: t.float().to(device)
+    outs = [torch.zeros(h.shape[0], w["w_out"].shape[0], dtype=torch.float64) for h in hs]
+    for items in schedule:
+        cu = [0]
+        for _, _, n in items:
+            cu.append(cu[-1] + n)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+        meta = AttnMeta(positions=i32([i for _, st, n in items for i in range(st, st + n)]), slots=i32([0]))
+        meta.seq_cu, meta.state_slots, meta.max_seq_len = i32(cu), i32([slots[s] for s, _, _ in items]), max(n for _, _, n in items)
+        h = dev(torch.cat([hs[s][st:st + n] for s, st, n in items]))
+        y = mamba2_mixer(h, dev(w["w_in"]), f32(w["conv_w"]), f32(w["conv_b"]), f32(w["dt_bias"]), f32(w["a_log"]),
+                         f32(w["d_skip"]), f32(w["norm_w"]), dev(w["w_out"]), spec, eps, (conv, ssm), meta).double().cpu()
+        r = 0
+        for s, st, n in items:
+            outs[s][st:st + n] = y[r:r + n]
+            r += n
+    return outs
+
+
+def oracle_mamba(spec, w, h, eps=1e-5):
+    return O.mamba2(h, w["w_in"], w["conv_w"], w["conv_b"], w["dt_bias"], w["a_log"], w["d_skip"], w["norm_w"], w["w_out"],
+                    spec.heads, spec.vdim, spec.state, spec.groups, spec.norm_groups, eps)
+
+
+MSPECS = [Mamba2Spec(4, 16, 16, 2, 4, 2), Mamba2Spec(3, 8, 24, 1, 2, 1), Mamba2Spec(2, 40, 72, 2, 3, 4),
+          Mamba2Spec(6, 4, 8, 6, 1, 3)]
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("spec", MSPECS, ids=lambda s: f"h{s.heads}p{s.vdim}n{s.state}g{s.groups}c{s.conv}")
+def test_mamba2_whole_chunked_decoded(spec, device, dtype):
+    """A whole sequence, the same cut into portions shorter than the convolution, and token by
+    token, beside a second sequence in another slot; slots start poisoned."""
+    g = torch.Generator().manual_seed(6)
+    W = 40
+    w = mamba_weights(g, spec, W)
+    hs = [q16(rnd(g, 33, W)), q16(rnd(g, 12, W))]
+    want = [oracle_mamba(spec, w, h) for h in hs]
+    whole = run_mamba(spec, w, hs, [[(0, 0, 33), (1, 0, 12)]], [2, 0], device, dtype)
+    sched = [[(0, 0, 1)], [(0, 1, 2), (1, 0, 5)], [(0, 3, 1), (1, 5, 1)], [(0, 4, 17), (1, 6, 2)], [(1, 8, 4)]] + \
+            [[(0, i, 1)] for i in range(21, 33)]
+    cut = run_mamba(spec, w, hs, sched, [3, 1], device, dtype)
+    for s in range(2):
+        assert rel_err(whole[s], want[s]) < tol(dtype)
+        assert rel_err(cut[s], want[s]) < tol(dtype)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_mamba2_slot_reuse_and_long_memory(device, dtype):
+    """A slot that held another sequence is taken by a new one (position 0 resets it); with a slow
+    decay the first token still shows after 200 single-token steps."""
+    g = torch.Generator().manual_seed(7)
+    spec, W = Mamba2Spec(2, 8, 16, 1, 4, 1), 24
+    w = mamba_weights(g, spec, W)
+    w["a_log"] = torch.tensor([-6.0, -5.0], dtype=torch.float64)     # decay exp(-dt e^-6) ~ 1
+    hs = [q16(rnd(g, 9, W)), q16(rnd(g, 201, W))]
+    want = oracle_mamba(spec, w, hs[1])
+    sched = [[(0, 0, 9)], [(1, 0, 1)]] + [[(1, i, 1)] for i in range(1, 201)]
+    got = run_mamba(spec, w, hs, sched, [1, 1], device, dtype, poison=False)[1]
+    assert rel_err(got, want) < tol(dtype) * 2
+    other = hs[1].clone()
+    other[0] = -other[0]
+    assert rel_err(oracle_mamba(spec, w, other)[200], want[200]) > 20 * tol(dtype)   # the test can see token 0
