@@ -272,10 +272,12 @@ __global__ __launch_bounds__(256) void sigattn_reduce_kernel(const float* __rest
 }
 
 // ---- unit-RMS q / k per head, k and v into the paged cache --------------------------------------
-// One workgroup per token; its 4 waves take the H + 2G (head, kind) jobs in turn.
+// One workgroup per token; its 4 waves take the H + 2G (head, kind) jobs in turn.  The mean of the
+// squares is over the head's first norm_dim elements' worth (norm_dim <= dim: heads padded with
+// zero columns up to the kernels' vector width keep their true size as the divisor).
 template <typename T>
 __global__ __launch_bounds__(256) void unitnorm_kv_write_kernel(T* __restrict__ qkv, long qs, int H, int G, int dim,
-                                                                int vdim, float eps, T* __restrict__ kc,
+                                                                int vdim, int norm_dim, float eps, T* __restrict__ kc,
                                                                 T* __restrict__ vc, const int* __restrict__ slots,
                                                                 int BS) {
   const long t = blockIdx.x;
@@ -293,7 +295,7 @@ __global__ __launch_bounds__(256) void unitnorm_kv_write_kernel(T* __restrict__ 
         ss += v * v;
       }
       ss = wave_sum(ss);
-      const float inv = 1.f / sqrtf(ss / (float)dim + eps);
+      const float inv = 1.f / sqrtf(ss / (float)norm_dim + eps);
       if (job < H) {
         for (int c = lane; c < dim; c += 64) El<T>::st(x + c, El<T>::ld(x + c) * inv);
       } else if (slot >= 0) {
@@ -377,15 +379,15 @@ SigParams make_params(const void* q, long qs, const void* kc, const void* vc, co
 
 int lk_sigattn_supported(int H, int G, int dim, int vdim, int BS, int esz) { return shape_ok(H, G, dim, vdim, BS, esz); }
 
-int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, float eps, void* kc, void* vc,
+int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, int norm_dim, float eps, void* kc, void* vc,
                          const int* slots, int BS, int esz, hipStream_t st) {
   if (T <= 0) return 0;
-  if (!shape_ok(H, G, dim, vdim, BS, esz)) return -1;
+  if (!shape_ok(H, G, dim, vdim, BS, esz) || norm_dim < 1 || norm_dim > dim) return -1;
   if (esz == 2)
-    unitnorm_kv_write_kernel<bf16_t><<<(unsigned)T, 256, 0, st>>>((bf16_t*)qkv, qs, H, G, dim, vdim, eps, (bf16_t*)kc,
+    unitnorm_kv_write_kernel<bf16_t><<<(unsigned)T, 256, 0, st>>>((bf16_t*)qkv, qs, H, G, dim, vdim, norm_dim, eps, (bf16_t*)kc,
                                                                   (bf16_t*)vc, slots, BS);
   else
-    unitnorm_kv_write_kernel<float><<<(unsigned)T, 256, 0, st>>>((float*)qkv, qs, H, G, dim, vdim, eps, (float*)kc,
+    unitnorm_kv_write_kernel<float><<<(unsigned)T, 256, 0, st>>>((float*)qkv, qs, H, G, dim, vdim, norm_dim, eps, (float*)kc,
                                                                  (float*)vc, slots, BS);
   LK_CHECK_LAUNCH();
   return 0;

@@ -1147,7 +1147,7 @@ void check_sig_caches(const at::Tensor& act, const at::Tensor& kc, const at::Ten
   TORCH_CHECK(reinterpret_cast<uintptr_t>(kc.data_ptr()) % 16 == 0 && reinterpret_cast<uintptr_t>(vc.data_ptr()) % 16 == 0, "cache alignment");
 }
 
-void unitnorm_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64_t vdim, double eps, at::Tensor& kc,
+void unitnorm_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64_t vdim, int64_t norm_dim, double eps, at::Tensor& kc,
                        at::Tensor& vc, const at::Tensor& slots) {
   CHECK_CUDA(qkv); CHECK_LASTDIM(qkv); CHECK_I32(slots); CHECK_CONTIG(slots);
   const int esz = esz_of(qkv, "qkv");
@@ -1157,7 +1157,7 @@ void unitnorm_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64
   const int BS = kc.size(2);
   const long nslots = kc.size(0) * BS;
   (void)nslots;
-  CHECK_RC(lk_unitnorm_kv_write(qkv.data_ptr(), qkv.stride(0), qkv.size(0), H, G, dim, vdim, (float)eps, kc.data_ptr(),
+  CHECK_RC(lk_unitnorm_kv_write(qkv.data_ptr(), qkv.stride(0), qkv.size(0), H, G, dim, vdim, norm_dim, (float)eps, kc.data_ptr(),
                                 vc.data_ptr(), ip(slots), BS, esz, cur_stream()), "unitnorm_kv_write");
 }
 

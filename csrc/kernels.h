@@ -230,7 +230,7 @@ int lk_softcap(const void* in, long is, float cap, float* out, long os, long row
 // csrc/attn_sigmoid.hip: sigmoid attention with a log-distance penalty (K cache [NB, G, BS, dim], V cache
 // [NB, G, vdim, BS])
 int lk_sigattn_supported(int H, int G, int dim, int vdim, int BS, int esz);
-int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, float eps, void* kc, void* vc,
+int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, int norm_dim, float eps, void* kc, void* vc,
                          const int* slots, int BS, int esz, hipStream_t st);
 int lk_sigattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride,
                        const int* cu_q, const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H,

@@ -175,11 +175,15 @@ class SigmoidAttnSpec:
     dim: int           # per-head q / k size
     vdim: int          # per-head v size
     scale: float
+    # the kernels read 16-byte fragments: a model whose head sizes are not multiples of 8 pads its
+    # projections with zero rows up to dim / vdim and names the true q / k size here (the divisor of
+    # the unit-RMS mean); 0 = dim
+    norm_dim: int = 0
 
     @classmethod
     def from_dict(cls, m: dict) -> "SigmoidAttnSpec":
         s = cls(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m.get("vdim", m["dim"])),
-                float(m.get("scale", int(m["dim"]) ** -0.5)))
+                float(m.get("scale", int(m["dim"]) ** -0.5)), int(m.get("norm_dim", 0)))
         if s.heads % s.kv_heads:
             raise ValueError(f"heads {s.heads} not a multiple of kv_heads {s.kv_heads}")
         return s
@@ -206,7 +210,7 @@ def sigmoid_paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta,
     T = qkv.shape[0]
     if out is None:
         out = torch.empty(T, H * vdim, dtype=qkv.dtype, device=qkv.device)
-    ops.unitnorm_kv_write(qkv, H, G, dim, vdim, eps, k_cache, v_cache, meta.slots)
+    ops.unitnorm_kv_write(qkv, H, G, dim, vdim, eps, k_cache, v_cache, meta.slots, norm_dim=spec.norm_dim or dim)
     Tp, Bd = meta.num_prefill_tokens, meta.num_decode
     if Tp:
         if meta.sig_tiles is None and qkv.is_cuda:

@@ -52,7 +52,9 @@ class LebepelLayer(nn.Module):
         self.type = spec.type
         self.norm1 = P(W, **f)
         if spec.type == "attention":
-            a = self.spec = SigmoidAttnSpec.from_dict(spec.mixer)
+            t = self.true = SigmoidAttnSpec.from_dict(spec.mixer)   # the checkpoint's sizes
+            # head sizes padded to the kernels' 8-element fragments with zero weight rows / columns
+            a = self.spec = SigmoidAttnSpec(t.heads, t.kv_heads, -(-t.dim // 8) * 8, -(-t.vdim // 8) * 8, t.scale, t.dim)
             self.qkv, self.qkv_b = P(a.qkv_out, W, **e), P(a.qkv_out, **e)
             self.o, self.o_b = P(W, a.heads * a.vdim, **e), P(W, **e)
             self.r1, self.r2, self.pb = P(a.heads, **f), P(a.heads, **f), P(a.heads, **f)
@@ -124,6 +126,15 @@ class LebepelModel(nn.Module):
                 rnd(p, i, 0.5)
             else:  # projections: unit-variance outputs for unit-variance inputs
                 rnd(p, i, 1.0 / math.sqrt(p.shape[1]))
+        for L in self.layers:
+            if L.type == "attention" and (L.spec.dim != L.true.dim or L.spec.vdim != L.true.vdim):
+                a, t = L.spec, L.true
+                k = 0
+                for h, d, dp in ((a.heads, t.dim, a.dim), (a.kv_heads, t.dim, a.dim), (a.kv_heads, t.vdim, a.vdim)):
+                    L.qkv[k:k + h * dp].view(h, dp, -1)[:, d:] = 0
+                    L.qkv_b[k:k + h * dp].view(h, dp)[:, d:] = 0
+                    k += h * dp
+                L.o.view(L.o.shape[0], a.heads, a.vdim)[:, :, t.vdim:] = 0
         return self
 
     @torch.no_grad()
@@ -144,9 +155,26 @@ class LebepelModel(nn.Module):
             put(L.norm1, b + "norm1")
             m = b + "mix."
             if L.type == "attention":
+                a, t = L.spec, L.true
+                parts = [(m + "q", a.heads, t.dim, a.dim), (m + "k", a.kv_heads, t.dim, a.dim), (m + "v", a.kv_heads, t.vdim, a.vdim)]
+                padded = dict(sd)
+                for n, h, d, dp in parts:  # [h * d, W] -> [h * dp, W], zero rows behind every head
+                    for key, tail in ((n, (sd[n].shape[1],)), (n + ".b", ())):
+                        if tuple(sd[key].shape) != (h * d, *tail):
+                            raise ValueError(f"{key}: checkpoint shape {tuple(sd[key].shape)} != {(h * d, *tail)}")
+                        z = torch.zeros(h, dp, *tail, dtype=sd[key].dtype)
+                        z[:, :d] = sd[key].view(h, d, *tail)
+                        padded[key] = z.view(h * dp, *tail)
+                if tuple(sd[m + "o"].shape) != (L.o.shape[0], a.heads * t.vdim):
+                    raise ValueError(f"{m}o: checkpoint shape {tuple(sd[m + 'o'].shape)}")
+                z = torch.zeros(L.o.shape[0], a.heads, a.vdim, dtype=sd[m + "o"].dtype)
+                z[:, :, :t.vdim] = sd[m + "o"].view(L.o.shape[0], a.heads, t.vdim)
+                padded[m + "o"] = z.view(L.o.shape[0], a.heads * a.vdim)
+                sd, keep = padded, sd
                 put(L.qkv, m + "q", m + "k", m + "v")
                 put(L.qkv_b, m + "q.b", m + "k.b", m + "v.b")
                 put(L.o, m + "o")
+                sd = keep
                 put(L.o_b, m + "o.b")
                 put(L.r1, m + "r1")
                 put(L.r2, m + "r2")
@@ -172,12 +200,15 @@ class LebepelModel(nn.Module):
             b, m = f"l{i}.", f"l{i}.mix."
             sd[b + "norm1"] = L.norm1
             if L.type == "attention":
-                a = L.spec
+                a, t = L.spec, L.true
                 nq, nk = a.heads * a.dim, a.kv_heads * a.dim
-                for n, w, bb in (("q", L.qkv[:nq], L.qkv_b[:nq]), ("k", L.qkv[nq:nq + nk], L.qkv_b[nq:nq + nk]),
-                                 ("v", L.qkv[nq + nk:], L.qkv_b[nq + nk:])):
-                    sd[m + n], sd[m + n + ".b"] = w, bb
-                sd.update({m + "o": L.o, m + "o.b": L.o_b, m + "r1": L.r1, m + "r2": L.r2, m + "pb": L.pb})
+                for n, w, bb, h, d, dp in (("q", L.qkv[:nq], L.qkv_b[:nq], a.heads, t.dim, a.dim),
+                                           ("k", L.qkv[nq:nq + nk], L.qkv_b[nq:nq + nk], a.kv_heads, t.dim, a.dim),
+                                           ("v", L.qkv[nq + nk:], L.qkv_b[nq + nk:], a.kv_heads, t.vdim, a.vdim)):
+                    sd[m + n] = w.view(h, dp, -1)[:, :d].reshape(h * d, -1)
+                    sd[m + n + ".b"] = bb.view(h, dp)[:, :d].reshape(h * d)
+                sd[m + "o"] = L.o.view(L.o.shape[0], a.heads, a.vdim)[:, :, :t.vdim].reshape(L.o.shape[0], -1)
+                sd.update({m + "o.b": L.o_b, m + "r1": L.r1, m + "r2": L.r2, m + "pb": L.pb})
             else:
                 sd.update({m + "in": L.in_proj, m + "conv": L.conv_w, m + "conv.b": L.conv_b, m + "dt_bias": L.dt_bias,
                            m + "A_log": L.A_log, m + "D": L.D, m + "norm": L.mix_norm, m + "o": L.o})

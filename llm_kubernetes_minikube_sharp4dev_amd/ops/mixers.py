@@ -89,15 +89,18 @@ def sigattn_supported(H: int, G: int, dim: int, vdim: int, block_size: int, dtyp
             and max(dim, vdim) <= SIG_MAX_HEAD)
 
 
-def unitnorm_kv_write(qkv, H: int, G: int, dim: int, vdim: int, eps: float, k_cache, v_cache, slots):
+def unitnorm_kv_write(qkv, H: int, G: int, dim: int, vdim: int, eps: float, k_cache, v_cache, slots,
+                      norm_dim: Optional[int] = None):
     """Rows ``[q: H dim | k: G dim | v: G vdim]``: q and k become x / sqrt(mean(x^2) + eps) per head
-    (f32 arithmetic; q in place, k into the cache), v goes into the cache.  Slots < 0 cache nothing."""
+    (f32 arithmetic; q in place, k into the cache), v goes into the cache.  Slots < 0 cache nothing.
+    ``norm_dim``: the divisor of the mean when the heads carry zero padding columns (default dim)."""
+    norm_dim = dim if norm_dim is None else int(norm_dim)
     if use_hip(qkv):
-        lib().unitnorm_kv_write(qkv, H, G, dim, vdim, float(eps), k_cache, v_cache, slots)
+        lib().unitnorm_kv_write(qkv, H, G, dim, vdim, norm_dim, float(eps), k_cache, v_cache, slots)
         return qkv
     T = qkv.shape[0]
     qk = qkv[:, : (H + G) * dim].float().view(T, H + G, dim)
-    qk = qk / torch.sqrt(qk.pow(2).mean(-1, keepdim=True) + eps)
+    qk = qk / torch.sqrt(qk.pow(2).sum(-1, keepdim=True) / norm_dim + eps)
     qkv[:, : (H + G) * dim] = qk.reshape(T, -1).to(qkv.dtype)
     BS = k_cache.shape[2]
     sl = slots[:T].long()

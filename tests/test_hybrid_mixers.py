@@ -322,10 +322,12 @@ def test_mamba2_slot_reuse_and_long_memory(device, dtype):
     w = mamba_weights(g, spec, W)
     w["a_log"] = torch.tensor([-6.0, -5.0], dtype=torch.float64)     # decay exp(-dt e^-6) ~ 1
     hs = [q16(rnd(g, 9, W)), q16(rnd(g, 201, W))]
+    hs[1][0] *= 4.0
     want = oracle_mamba(spec, w, hs[1])
     sched = [[(0, 0, 9)], [(1, 0, 1)]] + [[(1, i, 1)] for i in range(1, 201)]
     got = run_mamba(spec, w, hs, sched, [1, 1], device, dtype, poison=False)[1]
     assert rel_err(got, want) < tol(dtype) * 2
     other = hs[1].clone()
     other[0] = -other[0]
-    assert rel_err(oracle_mamba(spec, w, other)[200], want[200]) > 20 * tol(dtype)   # the test can see token 0
+    seen = rel_err(oracle_mamba(spec, w, other)[200], want[200])
+    assert seen > 5 * tol(dtype), seen   # the last row still depends on token 0: the comparison above sees a lost state
