@@ -133,6 +133,7 @@ class ModelRunner:
         # buckets up to twice the sequence cap: jump-forward extend chunks add decode rows
         self.graph_sizes = sorted(b for b in graph_batch_sizes if b <= 2 * max_num_seqs)
         self.graphs: dict = {}
+        self._eager_buckets: set = set()   # decode buckets that are not captured (capture())
         self._graph_pool = None
         self._ws = None
         self.step_hook = None
@@ -582,12 +583,23 @@ class ModelRunner:
         st = self._static(B)
         s = torch.cuda.Stream(self.device)
         s.wait_stream(torch.cuda.current_stream(self.device))
+        lib_calls = sum(ops.LIBRARY_FALLBACKS.values())
         with torch.cuda.stream(s):
             for _ in range(2):  # warm-up (allocator + lazy library init) outside capture
                 h = self.model(st["ids"], st["meta"], self.kv_caches)
                 self.model.greedy(h) if greedy else self.model.logits(h, dtype=self.logits_dtype)
         torch.cuda.current_stream(self.device).wait_stream(s)
         torch.cuda.synchronize(self.device)
+        if self.stateful and sum(ops.LIBRARY_FALLBACKS.values()) != lib_calls:
+            # a projection of this bucket runs on the vendor GEMM library (f32 activations, or a shape
+            # the MFMA kernels do not tile): library kernels may record memset nodes, which replay
+            # wrongly, so the bucket is not captured -- its steps run the same padded static inputs eagerly
+            if not self._eager_buckets:
+                log.info("decode bucket %d runs vendor GEMMs: not captured in a hipGraph (eager steps)", B)
+            self._eager_buckets.add((B, greedy))
+            st["graph"] = None
+            self.graphs[(B, greedy)] = st
+            return st
         if self._graph_pool is None:
             self._graph_pool = torch.cuda.graph_pool_handle()
         g = torch.cuda.CUDAGraph()
@@ -633,7 +645,11 @@ class ModelRunner:
             views = [None] + [torch.from_numpy(a).to(self.device, non_blocking=True) for a in arrays[1:]]
         if si.gather is not None:
             self._apply_gather(st["ids"], views[1], views[2])
-        st["graph"].replay()
+        if st["graph"] is None:  # a bucket that is not captured: the same static inputs, run eagerly
+            h = self.model(st["ids"], st["meta"], self.kv_caches)
+            st["logits"] = self.model.greedy(h) if si.greedy else self.model.logits(h, dtype=self.logits_dtype)
+        else:
+            st["graph"].replay()
         if subset:
             return ops.gather_rows(st["logits"], views[-1])
         return st["logits"][: si.num_decode]

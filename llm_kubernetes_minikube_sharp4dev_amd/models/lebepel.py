@@ -35,7 +35,7 @@ import torch.nn as nn
 from .. import ops
 from ..parallel.tp import SINGLE, TPGroup
 from .attention import AttnMeta, SigmoidAttnSpec, sigmoid_paged_attention
-from .configs import LebepelConfig
+from .configs import LebepelConfig, pad_vocab
 from .ssm import Mamba2Spec, mamba2_mixer
 
 
@@ -66,8 +66,9 @@ class LebepelLayer(nn.Module):
             self.mix_norm = P(s.inner, **f)
             self.o = P(W, s.inner, **e)
         self.ff = int(spec.mlp["ff"]) if spec.mlp else 0
+        self.ff_p = -(-self.ff // 8) * 8     # padded with zero gate / up rows and down columns (16-byte rows)
         if self.ff:
-            self.gate_up, self.down = P(2 * self.ff, W, **e), P(W, self.ff, **e)
+            self.gate_up, self.down = P(2 * self.ff_p, W, **e), P(W, self.ff_p, **e)
 
 
 class LebepelModel(nn.Module):
@@ -84,7 +85,9 @@ class LebepelModel(nn.Module):
         self.pos = nn.Parameter(torch.zeros(cfg.max_position, cfg.hidden, **e), requires_grad=False)
         self.layers = nn.ModuleList([LebepelLayer(cfg, l, dtype, device) for l in cfg.layers])
         self.final_norm = nn.Parameter(torch.zeros(cfg.hidden, dtype=torch.float32, device=device), requires_grad=False)
-        self.lm_head = nn.Parameter(torch.zeros(cfg.vocab_size, cfg.hidden, **e), requires_grad=False)
+        # head rows padded (zero rows) so that logits rows start 32-byte aligned for the sampling kernels;
+        # the padding columns are sliced off before anything reads the logits
+        self.lm_head = nn.Parameter(torch.zeros(pad_vocab(cfg.vocab_size, 64), cfg.hidden, **e), requires_grad=False)
         self.runs = cfg.layer_runs()
         self.reinject = any(add for _, add in self.runs)
         # the runner's attention workspaces are sized from these (largest attention layer)
@@ -135,6 +138,12 @@ class LebepelModel(nn.Module):
                     L.qkv_b[k:k + h * dp].view(h, dp)[:, d:] = 0
                     k += h * dp
                 L.o.view(L.o.shape[0], a.heads, a.vdim)[:, :, t.vdim:] = 0
+        for L in self.layers:
+            if L.ff != L.ff_p:
+                L.gate_up[L.ff:L.ff_p] = 0
+                L.gate_up[L.ff_p + L.ff:] = 0
+                L.down[:, L.ff:] = 0
+        self.lm_head[self.cfg.vocab_size:] = 0
         return self
 
     @torch.no_grad()
@@ -149,7 +158,10 @@ class LebepelModel(nn.Module):
         put(self.embed, "embed")
         put(self.pos, "pos")
         put(self.final_norm, "final.norm")
-        put(self.lm_head, "head")
+        if tuple(sd["head"].shape) != (self.cfg.vocab_size, self.cfg.hidden):
+            raise ValueError(f"head: checkpoint shape {tuple(sd['head'].shape)}")
+        self.lm_head.zero_()
+        self.lm_head[:self.cfg.vocab_size].copy_(sd["head"].to(self.lm_head.dtype))
         for i, L in enumerate(self.layers):
             b = f"l{i}."
             put(L.norm1, b + "norm1")
@@ -189,13 +201,20 @@ class LebepelModel(nn.Module):
                 put(L.mix_norm, m + "norm")
                 put(L.o, m + "o")
             if L.ff:
-                put(L.gate_up, b + "mlp.gate", b + "mlp.up")
-                put(L.down, b + "mlp.down")
+                g, u, dn = sd[b + "mlp.gate"], sd[b + "mlp.up"], sd[b + "mlp.down"]
+                if tuple(g.shape) != (L.ff, L.down.shape[0]) or g.shape != u.shape or tuple(dn.shape) != (L.down.shape[0], L.ff):
+                    raise ValueError(f"{b}mlp: checkpoint shapes {tuple(g.shape)}, {tuple(u.shape)}, {tuple(dn.shape)}")
+                L.gate_up.zero_()
+                L.down.zero_()
+                L.gate_up[:L.ff].copy_(g.to(L.gate_up.dtype))
+                L.gate_up[L.ff_p:L.ff_p + L.ff].copy_(u.to(L.gate_up.dtype))
+                L.down[:, :L.ff].copy_(dn.to(L.down.dtype))
         return self
 
     def native_state_dict(self) -> dict:
         """The inverse of :meth:`load_state_dict_native` (tests, export)."""
-        sd = {"embed": self.embed, "pos": self.pos, "final.norm": self.final_norm, "head": self.lm_head}
+        sd = {"embed": self.embed, "pos": self.pos, "final.norm": self.final_norm,
+              "head": self.lm_head[:self.cfg.vocab_size]}
         for i, L in enumerate(self.layers):
             b, m = f"l{i}.", f"l{i}.mix."
             sd[b + "norm1"] = L.norm1
@@ -213,7 +232,8 @@ class LebepelModel(nn.Module):
                 sd.update({m + "in": L.in_proj, m + "conv": L.conv_w, m + "conv.b": L.conv_b, m + "dt_bias": L.dt_bias,
                            m + "A_log": L.A_log, m + "D": L.D, m + "norm": L.mix_norm, m + "o": L.o})
             if L.ff:
-                sd[b + "mlp.gate"], sd[b + "mlp.up"], sd[b + "mlp.down"] = L.gate_up[:L.ff], L.gate_up[L.ff:], L.down
+                sd[b + "mlp.gate"], sd[b + "mlp.up"] = L.gate_up[:L.ff], L.gate_up[L.ff_p:L.ff_p + L.ff]
+                sd[b + "mlp.down"] = L.down[:, :L.ff]
         return {k: v.detach().clone().contiguous() for k, v in sd.items()}
 
     # ------------------------------------------------------------------ caches
@@ -275,10 +295,10 @@ class LebepelModel(nn.Module):
         return ops.stream_rmsnorm(x, a, b, None, m, self.final_norm, 1.0, eps, idx=meta.logits_idx, out_dtype=self.dtype)
 
     def head(self, hidden):
-        return ops.linear(hidden, self.lm_head)
+        return ops.linear(hidden, self.lm_head)[:, : self.cfg.vocab_size]
 
     def logits(self, hidden, gather: bool = True, dtype=torch.float32):
-        return ops.softcap(self.head(hidden), self.cfg.logit_softcap)
+        return ops.softcap(ops.linear(hidden, self.lm_head), self.cfg.logit_softcap)[:, : self.cfg.vocab_size]
 
     def greedy(self, hidden):
         # the cap is monotonic: the argmax of the raw head output is the argmax of the logits

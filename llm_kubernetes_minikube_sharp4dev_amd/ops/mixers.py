@@ -75,10 +75,10 @@ def softcap(z, cap: float):
 def linear_swiglu_any(x, w_gate_up):
     """silu(x Wg^T) * (x Wu^T) for a fused [Wg; Wu] weight in bf16 (the GEMM's SwiGLU epilogue) or,
     for f32 activations on the GPU, a true-f32 library product and an f32 activation kernel."""
-    from . import linear_swiglu
+    from . import _library, linear_swiglu
 
     if use_hip(x) and x.dtype == torch.float32:
-        return lib().silu_mul_f32(F.linear(x, w_gate_up))
+        return lib().silu_mul_f32(_library(x, w_gate_up, None, None, (True, w_gate_up.shape[0], w_gate_up.shape[1], 1)))
     return linear_swiglu(x, w_gate_up)
 
 
