@@ -140,7 +140,15 @@ def parse():
                     help="with --tp-sim: JSON of the measured per-call TP tail collective floor "
                          "(benchmarks/xgmi_floor.py --world 2; default profiles/r4_tp_collectives/floor_tp2_h<H>.json)")
     ap.add_argument("--json-out", default=None)
-    return ap.parse_args()
+    ap.add_argument("--decoder-bench", action="store_true",
+                    help="instead of the headline workload: prefill and decode tokens/s of the hybrid Lebepel decoder "
+                         "beside a Llama decoder of equal size at a few layer sizes (benchmarks/decoder_bench.py; "
+                         "its own options follow after --)")
+    args, rest = ap.parse_known_args()
+    if rest and not args.decoder_bench:
+        ap.error(f"unrecognized arguments: {' '.join(rest)}")
+    args.rest = [r for r in rest if r != "--"]
+    return args
 
 
 def log(rank, *a):
@@ -152,6 +160,12 @@ def main():
     args = parse()
     if args.admit_chunk is None:  # 1/8 of the in-flight requests per retrieval batch (16 at 128)
         args.admit_chunk = max(1, args.batch // 8)
+    if args.decoder_bench:  # a separate process, like --via-http: the headline contract below is untouched
+        import subprocess
+
+        cmd = [sys.executable, os.path.join(ROOT, "benchmarks", "decoder_bench.py")] + args.rest + \
+            (["--json-out", args.json_out] if args.json_out else [])
+        raise SystemExit(subprocess.call(cmd))
     if args.via_http:  # before any GPU use: the servers are child processes
         import subprocess
 

@@ -108,8 +108,13 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const T* __restrict__ u
 }
 
 // Sequential scan.  grid (sequence, head, P / 16): 256 threads = 16 state columns p x 16 slices of
-// the N state rows (thread holds rows ns, ns + 16, ...), so y_t[p] is a 16-lane butterfly.
-// The next token's operands are fetched while the current one is applied.
+// the N state rows (thread holds rows ns * NR .. ns * NR + NR - 1), so y_t[p] is a 16-lane butterfly.
+// Tokens are taken in tiles of kScanTile: the tile's B, C (as f32), x, softplus(dt) and the decay are
+// staged in LDS with coalesced loads (16-byte ones when the row layout allows), so the recurrence
+// itself runs on LDS reads only -- per-token global loads of a few bytes per lane made the first
+// version address-unit bound (18 tiny loads per lane and token).
+constexpr int kScanTile = 16;
+
 template <typename T, int NR>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc, long xs, const T* __restrict__ dtp,
                                                        long dts, int heads, int P, int N, int groups,
@@ -119,68 +124,99 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
                                                        const int* __restrict__ slots,
                                                        const int* __restrict__ positions, float* __restrict__ y,
                                                        long ys) {
-  const int s = blockIdx.x, h = blockIdx.y;
-  const int ns = threadIdx.x & 15, p = blockIdx.z * 16 + (threadIdx.x >> 4);
+  constexpr int NP = NR * 16;  // padded state rows
+  constexpr int EV = 16 / sizeof(T);
+  __shared__ __attribute__((aligned(16))) float sB[kScanTile][NP];
+  __shared__ __attribute__((aligned(16))) float sC[kScanTile][NP];
+  __shared__ float sx[kScanTile][16], sy[kScanTile][16], sdt[kScanTile], sdA[kScanTile];
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int ns = tid & 15, pl = tid >> 4, p0 = blockIdx.z * 16, p = p0 + pl;
   const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
   if (len <= 0) return;
   const bool pv = p < P;
   if (slot < 0) {
-    if (pv && ns == 0)
-      for (int i = 0; i < len; ++i) y[(long)(row0 + i) * ys + (long)h * P + p] = 0.f;
+    for (int i = tid; i < len * 16; i += 256)
+      if (p0 + (i & 15) < P) y[(long)(row0 + (i >> 4)) * ys + (long)h * P + p0 + (i & 15)] = 0.f;
     return;
   }
   const int inner = heads * P, grp = h / (heads / groups);
-  const long xo = (long)h * P + (pv ? p : 0), bo = inner + (long)grp * N, co = inner + (long)groups * N + (long)grp * N;
+  const long xo = (long)h * P + p0, bo = inner + (long)grp * N, co = inner + (long)groups * N + (long)grp * N;
   float* sp = state + (((long)slot * heads + h) * P + (pv ? p : 0)) * N;
   float S[NR];
   const bool past = positions[row0] > 0;
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
-    const int n = ns + 16 * i;
+    const int n = ns * NR + i;
     S[i] = (past && pv && n < N) ? sp[n] : 0.f;
   }
   const float nA = -expf(A_log[h]), db = dt_bias[h], Dh = Dp[h];
-  float Bn[NR], Cn[NR], xv, dtr;
-  auto fetch = [&](int i, float (&B)[NR], float (&Cc)[NR], float& x, float& d) {
-    const T* r = xbc + (long)(row0 + i) * xs;
-    x = ldf<T>(r + xo);
-    d = ldf<T>(dtp + (long)(row0 + i) * dts + h);
+  // 16-byte staging loads need every row's B / C run to start on a 16-byte boundary
+  const bool vec = N % EV == 0 && xs % EV == 0 && bo % EV == 0 && co % EV == 0 &&
+                   (reinterpret_cast<uintptr_t>(xbc) & 15) == 0;
+  for (int t0 = 0; t0 < len; t0 += kScanTile) {
+    const int tl = min(kScanTile, len - t0);
+    __syncthreads();  // the previous tile's sy / sB readers are done
+    if (vec) {
+      const int cpr = N / EV;  // 16-byte chunks per row
+      for (int i = tid; i < tl * cpr * 2; i += 256) {
+        const int which = i / (tl * cpr), r = i % (tl * cpr), t = r / cpr, c = r % cpr;
+        const T* src = xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + c * EV;
+        float* dst = (which ? sC[t] : sB[t]) + c * EV;
+        if constexpr (sizeof(T) == 2) {
+          const short8 v = *reinterpret_cast<const short8*>(src);
 #pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      const int n = ns + 16 * k;
-      B[k] = n < N ? ldf<T>(r + bo + n) : 0.f;
-      Cc[k] = n < N ? ldf<T>(r + co + n) : 0.f;
+          for (int e = 0; e < 8; ++e) dst[e] = bf2f((bf16_t)v[e]);
+        } else {
+          *reinterpret_cast<floatx4*>(dst) = *reinterpret_cast<const floatx4*>(src);
+        }
+      }
+    } else {
+      for (int i = tid; i < tl * N * 2; i += 256) {
+        const int which = i / (tl * N), r = i % (tl * N), t = r / N, n = r % N;
+        (which ? sC[t] : sB[t])[n] = ldf<T>(xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + n);
+      }
     }
-  };
-  fetch(0, Bn, Cn, xv, dtr);
-  for (int i = 0; i < len; ++i) {
-    float B[NR], Cc[NR];
-    const float x = xv, dr = dtr;
+    if (N < NP)
+      for (int i = tid; i < tl * (NP - N); i += 256) {
+        const int t = i / (NP - N), n = N + i % (NP - N);
+        sB[t][n] = 0.f;
+        sC[t][n] = 0.f;
+      }
+    {
+      const int t = tid >> 4, c = tid & 15;  // 16 tokens x 16 columns: one x each
+      if (t < tl) sx[t][c] = p0 + c < P ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + xo + c) : 0.f;
+      if (tid < tl) {
+        const float a = ldf<T>(dtp + (long)(row0 + t0 + tid) * dts + h) + db;
+        const float dt = a > 20.f ? a : log1pf(expf(a));
+        sdt[tid] = dt;
+        sdA[tid] = expf(nA * dt);
+      }
+    }
+    __syncthreads();
+    for (int t = 0; t < tl; ++t) {
+      const float x = sx[t][pl], dA = sdA[t], dx = sdt[t] * x;
+      float acc = 0.f;
 #pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      B[k] = Bn[k];
-      Cc[k] = Cn[k];
+      for (int k = 0; k < NR; ++k) {
+        S[k] = dA * S[k] + dx * sB[t][ns * NR + k];
+        acc += S[k] * sC[t][ns * NR + k];
+      }
+      acc += __shfl_xor(acc, 1, 64);
+      acc += __shfl_xor(acc, 2, 64);
+      acc += __shfl_xor(acc, 4, 64);
+      acc += __shfl_xor(acc, 8, 64);
+      if (ns == 0) sy[t][pl] = acc + Dh * x;
     }
-    if (i + 1 < len) fetch(i + 1, Bn, Cn, xv, dtr);
-    const float a = dr + db;
-    const float dt = a > 20.f ? a : log1pf(expf(a));
-    const float dA = expf(nA * dt), dx = dt * x;
-    float acc = 0.f;
-#pragma unroll
-    for (int k = 0; k < NR; ++k) {
-      S[k] = dA * S[k] + dx * B[k];
-      acc += S[k] * Cc[k];
+    __syncthreads();
+    {
+      const int t = tid >> 4, c = tid & 15;
+      if (t < tl && p0 + c < P) y[(long)(row0 + t0 + t) * ys + (long)h * P + p0 + c] = sy[t][c];
     }
-    acc += __shfl_xor(acc, 1, 64);
-    acc += __shfl_xor(acc, 2, 64);
-    acc += __shfl_xor(acc, 4, 64);
-    acc += __shfl_xor(acc, 8, 64);
-    if (pv && ns == 0) y[(long)(row0 + i) * ys + (long)h * P + p] = acc + Dh * x;
   }
   if (pv) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-      const int n = ns + 16 * i;
+      const int n = ns * NR + i;
       if (n < N) sp[n] = S[i];
     }
   }

@@ -60,7 +60,8 @@ class LebepelLayer(nn.Module):
             self.r1, self.r2, self.pb = P(a.heads, **f), P(a.heads, **f), P(a.heads, **f)
         else:
             s = self.spec = Mamba2Spec.from_dict(spec.mixer)
-            self.in_proj = P(s.proj_out, W, **e)
+            # rows [z | x B C | dt], padded with zero rows to the decode GEMMs' 128-column tiles
+            self.in_proj = P(-(-s.proj_out // 128) * 128, W, **e)
             self.conv_w, self.conv_b = P(s.conv_channels, s.conv, **f), P(s.conv_channels, **f)
             self.dt_bias, self.A_log, self.D = P(s.heads, **f), P(s.heads, **f), P(s.heads, **f)
             self.mix_norm = P(s.inner, **f)
@@ -144,6 +145,9 @@ class LebepelModel(nn.Module):
                 L.gate_up[L.ff_p + L.ff:] = 0
                 L.down[:, L.ff:] = 0
         self.lm_head[self.cfg.vocab_size:] = 0
+        for L in self.layers:
+            if L.type == "mamba2":
+                L.in_proj[L.spec.proj_out:] = 0
         return self
 
     @torch.no_grad()
@@ -192,7 +196,10 @@ class LebepelModel(nn.Module):
                 put(L.r2, m + "r2")
                 put(L.pb, m + "pb")
             else:
-                put(L.in_proj, m + "in")
+                if tuple(sd[m + "in"].shape) != (L.spec.proj_out, L.in_proj.shape[1]):
+                    raise ValueError(f"{m}in: checkpoint shape {tuple(sd[m + 'in'].shape)}")
+                L.in_proj.zero_()
+                L.in_proj[:L.spec.proj_out].copy_(sd[m + "in"].to(L.in_proj.dtype))
                 put(L.conv_w, m + "conv")
                 put(L.conv_b, m + "conv.b")
                 put(L.dt_bias, m + "dt_bias")
@@ -229,12 +236,28 @@ class LebepelModel(nn.Module):
                 sd[m + "o"] = L.o.view(L.o.shape[0], a.heads, a.vdim)[:, :, :t.vdim].reshape(L.o.shape[0], -1)
                 sd.update({m + "o.b": L.o_b, m + "r1": L.r1, m + "r2": L.r2, m + "pb": L.pb})
             else:
-                sd.update({m + "in": L.in_proj, m + "conv": L.conv_w, m + "conv.b": L.conv_b, m + "dt_bias": L.dt_bias,
+                sd.update({m + "in": L.in_proj[:L.spec.proj_out], m + "conv": L.conv_w, m + "conv.b": L.conv_b, m + "dt_bias": L.dt_bias,
                            m + "A_log": L.A_log, m + "D": L.D, m + "norm": L.mix_norm, m + "o": L.o})
             if L.ff:
                 sd[b + "mlp.gate"], sd[b + "mlp.up"] = L.gate_up[:L.ff], L.gate_up[L.ff_p:L.ff_p + L.ff]
                 sd[b + "mlp.down"] = L.down[:, :L.ff]
         return {k: v.detach().clone().contiguous() for k, v in sd.items()}
+
+    def decode_gemm_shapes(self):
+        """(weight, swiglu) of the bias-free projections a decode step runs, one per distinct shape, for
+        the engine's decode GEMM routing (ops.tune_decode)."""
+        if self.dtype != torch.bfloat16:
+            return []   # f32 activations run on the vendor library: nothing to route
+        seen, out = set(), []
+        for L in self.layers:
+            ws = [(L.in_proj, False), (L.o, False)] if L.type == "mamba2" else []
+            ws += [(L.gate_up, True), (L.down, False)] if L.ff else []
+            for w, sw in ws:
+                if (tuple(w.shape), sw) not in seen:
+                    seen.add((tuple(w.shape), sw))
+                    out.append((w, sw))
+        # (weights too small to matter are left to the static rule: the tuner streams each from cold HBM copies)
+        return [(w, sw) for w, sw in out + [(self.lm_head, False)] if w.numel() >= 1 << 20]
 
     # ------------------------------------------------------------------ caches
     def make_caches(self, num_blocks: int, block_size: int, num_slots: int) -> list:

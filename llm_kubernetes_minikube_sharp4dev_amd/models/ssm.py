@@ -64,7 +64,7 @@ def mamba2_mixer(h, w_in, conv_w, conv_b, dt_bias, A_log, D, norm_w, w_out, spec
     inner, C = spec.inner, spec.conv_channels
     xbc = ops.conv_silu(u, inner, C, conv_w, conv_b, conv_state, meta.seq_cu, meta.state_slots, meta.positions,
                         meta.max_seq_len)
-    y = ops.ssm_scan(xbc, u[:, inner + C:], spec.heads, spec.vdim, spec.state, spec.groups, dt_bias, A_log, D,
+    y = ops.ssm_scan(xbc, u[:, inner + C:inner + C + spec.heads], spec.heads, spec.vdim, spec.state, spec.groups, dt_bias, A_log, D,
                      ssm_state, meta.seq_cu, meta.state_slots, meta.positions)
     g = ops.gated_group_rmsnorm(y, u[:, :inner], norm_w, spec.norm_groups, eps)
     return ops.linear(g, w_out)
