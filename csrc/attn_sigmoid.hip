@@ -85,46 +85,71 @@ LK_DEVICE float sig_weight(float s, float r1, float r2, float pb, int d) {
 // The columns of this wave against the 32-key steps step0, step0 + stride, ... of keys [k0, k1):
 // k0 is a multiple of 32; k1 <= the sequence's context.  Column n = lane % 16 sits at position
 // qpos and sees keys <= qpos.
+//
+// Key order inside a step: row m of S^T tile t is key 8 (m / 4) + 4 t + m % 4, so after both tiles
+// lane group g holds the weights of the 8 CONSECUTIVE keys 8g .. 8g + 7 -- one 16-byte piece of a
+// V^T row (bf16), and exactly the k-slots 8g .. 8g + 7 of the P.V MFMA's B operand.  Keys at or
+// past k1 are read from the last valid key / key run (always allocated, finite) and weigh zero.
+// bf16: the next step's K fragments are requested as soon as this step's Q.K MFMAs have
+// consumed the current ones, and this step's V fragments before the weights are computed, so
+// both fly under the transcendental-heavy weight arithmetic.
 template <typename T, int PAD>
 LK_DEVICE void sig_run(const SigParams& p, const uint4_t (&qf)[PAD / (4 * El<T>::V)], int kvh, const int* bt, int k0,
                        int k1, int step0, int stride, bool cvalid, int qpos, float r1, float r2, float pb,
                        floatx4 (&o)[PAD / 16]) {
   constexpr int EV = El<T>::V, KS = PAD / (4 * EV), VT = PAD / 16;
+  constexpr bool PIPE = sizeof(T) == 2;
   const int lane = threadIdx.x & 63, n16 = lane & 15, g = lane >> 4;
   const T* kc = reinterpret_cast<const T*>(p.kc);
   const T* vc = reinterpret_cast<const T*>(p.vc);
-  for (int kb = k0 + 32 * step0; kb < k1; kb += 32 * stride) {
-    float pw[2][4];
-    const T* vrow[2];
-    bool tv[2];
+  const int krow = 8 * (n16 >> 2) + (n16 & 3);  // this lane's K row inside a step (+ 4 t)
+  auto load_k = [&](int kb, uint4_t (&kf)[2][KS]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int kt = kb + 16 * t;
-      tv[t] = kt < k1;
-      vrow[t] = vc;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) pw[t][j] = 0.f;
-      if (!tv[t]) continue;
-      const int blk = bt[kt / p.BS], off = kt % p.BS;
-      const T* kr = kc + (((long)blk * p.G + kvh) * p.BS + off + n16) * p.dim;
-      vrow[t] = vc + ((long)blk * p.G + kvh) * p.vdim * p.BS + off + 4 * g;
-      floatx4 c = {0.f, 0.f, 0.f, 0.f};
+      const int key = min(kb + krow + 4 * t, k1 - 1);
+      const T* kr = kc + (((long)bt[key / p.BS] * p.G + kvh) * p.BS + key % p.BS) * p.dim;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const int d0 = s * 4 * EV + g * EV;
-        if (s * 4 * EV < p.dim) {
-          const uint4_t a = d0 < p.dim ? ld16(kr + d0) : uint4_t{0u, 0u, 0u, 0u};
-          c = mma_qk<T>(a, qf[s], c);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int key = kt + 4 * g + j, d = qpos - key;
-        if (cvalid && d >= 0 && key < k1) pw[t][j] = sig_weight<sizeof(T) == 4>(c[j] * p.scale, r1, r2, pb, d);
+        kf[t][s] = d0 < p.dim ? ld16(kr + d0) : uint4_t{0u, 0u, 0u, 0u};
       }
     }
-    if constexpr (sizeof(T) == 2) {
-      // one k-step of 32 keys: lane group g brings keys {4g + j} of the first tile and {16 + 4g + j} of the second
+  };
+  uint4_t kf[2][KS];
+  int kb = k0 + 32 * step0;
+  if (PIPE && kb < k1) load_k(kb, kf);
+  for (; kb < k1; kb += 32 * stride) {
+    if (!PIPE) load_k(kb, kf);
+    floatx4 c[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      c[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        if (s * 4 * EV < p.dim) c[t] = mma_qk<T>(kf[t][s], qf[s], c[t]);
+    }
+    // this lane group's run of 8 keys of V^T (a masked run re-reads the last valid one)
+    const int vk = kb + 8 * g < k1 ? kb + 8 * g : ((k1 - 1) & ~7);
+    const T* vrow = vc + ((long)bt[vk / p.BS] * p.G + kvh) * p.vdim * p.BS + vk % p.BS;
+    uint4_t vf[PIPE ? VT : 1];
+    if constexpr (PIPE) {
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        const int vd = vt * 16 + n16;
+        vf[vt] = (vt * 16 < p.vdim && vd < p.vdim) ? ld16(vrow + (long)vd * p.BS) : uint4_t{0u, 0u, 0u, 0u};
+      }
+      const int kn = kb + 32 * stride;
+      if (kn < k1) load_k(kn, kf);
+    }
+    float pw[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int key = kb + 8 * g + 4 * t + j, d = qpos - key;
+        pw[t][j] = (cvalid && d >= 0 && key < k1) ? sig_weight<sizeof(T) == 4>(c[t][j] * p.scale, r1, r2, pb, d) : 0.f;
+      }
+    if constexpr (PIPE) {
       short8 pbits;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -132,28 +157,18 @@ LK_DEVICE void sig_run(const SigParams& p, const uint4_t (&qf)[PAD / (4 * El<T>:
         pbits[4 + j] = (short)f2bf(pw[1][j]);
       }
 #pragma unroll
+      for (int vt = 0; vt < VT; ++vt)
+        if (vt * 16 < p.vdim)
+          o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(short8, vf[vt]), pbits, o[vt], 0, 0, 0);
+    } else {
+#pragma unroll
       for (int vt = 0; vt < VT; ++vt) {
         if (vt * 16 < p.vdim) {
           const int vd = vt * 16 + n16;
-          short4_t lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-          if (vd < p.vdim) {
-            if (tv[0]) lo = *reinterpret_cast<const short4_t*>(vrow[0] + (long)vd * p.BS);
-            if (tv[1]) hi = *reinterpret_cast<const short4_t*>(vrow[1] + (long)vd * p.BS);
-          }
-          const short8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pbits, o[vt], 0, 0, 0);
-        }
-      }
-    } else {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        if (!tv[t]) continue;
-#pragma unroll
-        for (int vt = 0; vt < VT; ++vt) {
-          if (vt * 16 < p.vdim) {
-            const int vd = vt * 16 + n16;
+          for (int t = 0; t < 2; ++t) {
             floatx4 a = {0.f, 0.f, 0.f, 0.f};
-            if (vd < p.vdim) a = *reinterpret_cast<const floatx4*>(vrow[t] + (long)vd * p.BS);
+            if (vd < p.vdim) a = *reinterpret_cast<const floatx4*>(vrow + (long)vd * p.BS + 4 * t);
 #pragma unroll
             for (int j = 0; j < 4; ++j) o[vt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], pw[t][j], o[vt], 0, 0, 0);
           }
