@@ -189,7 +189,30 @@ LK_DEVICE void load_q(const SigParams& p, const T* qrow, bool cvalid, uint4_t (&
   }
 }
 
-// ---- prefill: workgroup = 4 waves = 4 heads of one 16-query tile -------------------------------
+// Sum of the 4 waves' O^T accumulators in wave order through LDS; afterwards wave 0 holds the total.
+template <int VT>
+LK_DEVICE void sum_waves(floatx4 (&o)[VT], float (&red)[3][VT][64][4]) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (w > 0) {
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) red[w - 1][vt][lane][j] = o[vt][j];
+  }
+  __syncthreads();
+  if (w == 0) {
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[vt][j] = ((o[vt][j] + red[0][vt][lane][j]) + red[1][vt][lane][j]) + red[2][vt][lane][j];
+  }
+}
+
+// ---- prefill: workgroup = one 16-query tile of one head; its 4 waves take every fourth 32-key
+// step of the tile's causal key range and are summed through LDS.  (Four heads per workgroup, one
+// wave each, left a long row's 30-odd dependent steps on one wave: the kernel was bound by that
+// chain, not by arithmetic.)  blockIdx.x = head, so the heads of a kv group that read the same K / V
+// run side by side; blockIdx.y walks the host's tile list, heaviest tiles first.
 template <typename T, int PAD>
 __global__ __launch_bounds__(256) void sigattn_prefill_kernel(SigParams p, const int* __restrict__ cu_q,
                                                               const int* __restrict__ ctx_lens,
@@ -197,10 +220,10 @@ __global__ __launch_bounds__(256) void sigattn_prefill_kernel(SigParams p, const
                                                               const int* __restrict__ tile_q0, T* __restrict__ out,
                                                               long os) {
   constexpr int VT = PAD / 16;
+  __shared__ float red[3][VT][64][4];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, n16 = lane & 15, g = lane >> 4;
-  const int head = blockIdx.y * 4 + w;
-  if (head >= p.H) return;
-  const int b = tile_seq[blockIdx.x], q0 = tile_q0[blockIdx.x];
+  const int head = blockIdx.x;
+  const int b = tile_seq[blockIdx.y], q0 = tile_q0[blockIdx.y];
   const int qbeg = cu_q[b], qlen = cu_q[b + 1] - qbeg, ctx = ctx_lens[b], past = ctx - qlen;
   const int qi = q0 + n16;
   const bool cvalid = qi < qlen;
@@ -212,9 +235,10 @@ __global__ __launch_bounds__(256) void sigattn_prefill_kernel(SigParams p, const
 #pragma unroll
   for (int vt = 0; vt < VT; ++vt) o[vt] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int k1 = min(ctx, past + q0 + 16);
-  sig_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, k1, 0, 1, cvalid, qpos, p.r1[head],
+  sig_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, k1, w, 4, cvalid, qpos, p.r1[head],
                   p.r2[head], p.pb[head], o);
-  if (cvalid) {
+  sum_waves<VT>(o, red);
+  if (w == 0 && cvalid) {
     T* orow = out + (long)(qbeg + qi) * os + (long)head * p.vdim;
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt)
@@ -252,13 +276,7 @@ __global__ __launch_bounds__(256) void sigattn_decode_kernel(SigParams p, const 
   if (s0 < s1)
     sig_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, 32 * s0, min(ctx, 32 * s1), w, 4, cvalid, ctx - 1,
                     p.r1[head], p.r2[head], p.pb[head], o);
-  if (w > 0) {
-#pragma unroll
-    for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) red[w - 1][vt][lane][j] = o[vt][j];
-  }
-  __syncthreads();
+  sum_waves<VT>(o, red);
   if (w == 0 && cvalid) {
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt)
@@ -266,9 +284,8 @@ __global__ __launch_bounds__(256) void sigattn_decode_kernel(SigParams p, const 
       for (int j = 0; j < 4; ++j) {
         const int vd = vt * 16 + 4 * g + j;
         if (vd < p.vdim) {
-          const float v = ((o[vt][j] + red[0][vt][lane][j]) + red[1][vt][lane][j]) + red[2][vt][lane][j];
-          if (Z == 1) El<T>::st(out + (long)b * os + (long)head * p.vdim + vd, v);
-          else part[(((long)b * p.H + head) * Z + z) * p.vdim + vd] = v;
+          if (Z == 1) El<T>::st(out + (long)b * os + (long)head * p.vdim + vd, o[vt][j]);
+          else part[(((long)b * p.H + head) * Z + z) * p.vdim + vd] = o[vt][j];
         }
       }
   }
@@ -340,7 +357,8 @@ bool shape_ok(int H, int G, int dim, int vdim, int BS, int esz) {
 template <typename T, int PAD>
 int launch_prefill(const SigParams& p, const int* cu_q, const int* ctx, const int* ts, const int* tq, int ntiles,
                    void* out, long os, hipStream_t st) {
-  dim3 grid(ntiles, (p.H + 3) / 4);
+  if (ntiles > 65535) return -2;
+  dim3 grid(p.H, ntiles);
   sigattn_prefill_kernel<T, PAD><<<grid, 256, 0, st>>>(p, cu_q, ctx, ts, tq, reinterpret_cast<T*>(out), os);
   LK_CHECK_LAUNCH();
   return 0;

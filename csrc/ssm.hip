@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
     }
     __syncthreads();
     if (vec && t0 + kScanTile < len) fetch(t0 + kScanTile);
-    for (int t = 0; t < tl; ++t) {
+    auto token = [&](int t) {
       const float x = sx[t][pl], dA = sdA[t], dx = sdt[t] * x;
       float acc = 0.f;
 #pragma unroll
@@ -232,6 +232,12 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
       acc += __shfl_xor(acc, 4, 64);
       acc += __shfl_xor(acc, 8, 64);
       if (ns == 0) sy[t][pl] = acc + Dh * x;
+    };
+    if (tl == kScanTile) {  // whole tile: unrolled, so a token's LDS reads issue under its predecessor's reduction
+#pragma unroll
+      for (int t = 0; t < kScanTile; ++t) token(t);
+    } else {
+      for (int t = 0; t < tl; ++t) token(t);
     }
     __syncthreads();
     {

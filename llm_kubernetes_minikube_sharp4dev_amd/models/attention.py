@@ -214,7 +214,7 @@ def sigmoid_paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta,
     Tp, Bd = meta.num_prefill_tokens, meta.num_decode
     if Tp:
         if meta.sig_tiles is None and qkv.is_cuda:
-            ts, tq = ops.sig_prefill_tiles(meta.q_lens_cpu)
+            ts, tq = ops.sig_prefill_tiles(meta.q_lens_cpu, meta.ctx_lens_cpu)
             meta.sig_tiles = (torch.from_numpy(ts).to(qkv.device, non_blocking=True),
                               torch.from_numpy(tq).to(qkv.device, non_blocking=True))
         ops.sigmoid_attention_prefill(qkv[:Tp], k_cache, v_cache, meta.block_tables_p, meta.cu_q, meta.ctx_lens_p,

@@ -111,15 +111,15 @@ def unitnorm_kv_write(qkv, H: int, G: int, dim: int, vdim: int, eps: float, k_ca
     return qkv
 
 
-def sig_prefill_tiles(q_lens: Sequence[int]):
-    """(tile_seq, tile_q0) int32: one entry per 16-query tile of each chunk; a tile's cost grows with
-    its position in the sequence, so the later tiles of a chunk are listed (and start) first."""
-    seq, q0 = [], []
+def sig_prefill_tiles(q_lens: Sequence[int], ctx_lens: Optional[Sequence[int]] = None):
+    """(tile_seq, tile_q0) int32: one entry per 16-query tile of each chunk, heaviest first -- a tile
+    attends every key up to its last query, so its cost is its end position in the sequence."""
+    tiles = []
     for b, n in enumerate(q_lens):
-        for s in range(((n + SIG_TILE_ROWS - 1) // SIG_TILE_ROWS - 1) * SIG_TILE_ROWS, -1, -SIG_TILE_ROWS):
-            seq.append(b)
-            q0.append(s)
-    return np.asarray(seq, dtype=np.int32), np.asarray(q0, dtype=np.int32)
+        past = (ctx_lens[b] - n) if ctx_lens is not None else 0
+        tiles += [(past + s + SIG_TILE_ROWS, b, s) for s in range(0, n, SIG_TILE_ROWS)]
+    tiles.sort(key=lambda t: -t[0])
+    return (np.asarray([t[1] for t in tiles], dtype=np.int32), np.asarray([t[2] for t in tiles], dtype=np.int32))
 
 
 def sig_decode_splits(B: int, G: int, rep: int, max_context: int) -> int:
@@ -159,7 +159,7 @@ def sigmoid_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens,
     if use_hip(q):
         if tiles is None:
             ql = q_lens_cpu if q_lens_cpu is not None else (cu_q[1:] - cu_q[:-1]).tolist()
-            ts, tq = sig_prefill_tiles(ql)
+            ts, tq = sig_prefill_tiles(ql, ctx_lens.tolist())
             tiles = (torch.from_numpy(ts).to(q.device), torch.from_numpy(tq).to(q.device))
         lib().sigattn_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, tiles[0], tiles[1], H, G, dim, vdim,
                               float(scale), r1, r2, pb, out)
