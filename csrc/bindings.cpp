@@ -1235,7 +1235,7 @@ at::Tensor conv_silu(const at::Tensor& u, int64_t col0, int64_t C, const at::Ten
 // xbc: [T, heads P + 2 groups N] = [x | B | C] after the convolution; dt: [T, heads] view (row-strided)
 at::Tensor ssm_scan(const at::Tensor& xbc, const at::Tensor& dt, int64_t heads, int64_t P, int64_t N, int64_t groups,
                     const at::Tensor& dt_bias, const at::Tensor& A_log, const at::Tensor& D, at::Tensor& state,
-                    const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& positions) {
+                    const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& positions, int64_t max_len) {
   CHECK_CUDA(xbc); CHECK_LASTDIM(xbc); CHECK_LASTDIM(dt);
   const int esz = esz_of(xbc, "xbc");
   same_type(dt, xbc, "dt");
@@ -1246,7 +1246,7 @@ at::Tensor ssm_scan(const at::Tensor& xbc, const at::Tensor& dt, int64_t heads, 
   at::Tensor y = at::empty({xbc.size(0), heads * P}, xbc.options().dtype(at::kFloat));
   CHECK_RC(lk_ssm_scan(xbc.data_ptr(), xbc.stride(0), dt.data_ptr(), dt.stride(0), cu.numel() - 1, heads, P, N, groups,
                        fp(dt_bias, heads, "dt_bias"), fp(A_log, heads, "A_log"), fp(D, heads, "D"), state.data_ptr<float>(),
-                       ip(cu), ip(slots), ip(positions), y.data_ptr<float>(), y.stride(0), esz, cur_stream()), "ssm_scan");
+                       ip(cu), ip(slots), ip(positions), y.data_ptr<float>(), y.stride(0), (int)max_len, esz, cur_stream()), "ssm_scan");
   return y;
 }
 

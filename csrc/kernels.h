@@ -247,6 +247,6 @@ int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const 
                  hipStream_t st);
 int lk_ssm_scan(const void* xbc, long xs, const void* dt, long dts, int S, int heads, int P, int N, int groups,
                 const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
-                const int* positions, float* y, long ys, int esz, hipStream_t st);
+                const int* positions, float* y, long ys, int max_len, int esz, hipStream_t st);
 int lk_gated_group_rmsnorm(const float* y, long ys, const void* z, long zs, const float* w, long rows, int inner,
                            int ngroups, float eps, void* out, long os, int esz, hipStream_t st);

@@ -254,6 +254,170 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const T* __restrict__ xbc
   }
 }
 
+// Chunked (matrix-form) scan for prompt portions: the recurrence is unrolled over chunks of 16
+// tokens and every product runs on true-f32 MFMAs (v_mfma_f32_16x16x4_f32), the state staying in
+// the accumulators' layout from chunk to chunk.  With a_t = -exp(A_log) dt_t, c_t = a_1 + .. + a_t
+// inside the chunk and S the state before it:
+//   y_t  = exp(c_t) C_t^T S  +  sum_{s<=t} exp(c_t - c_s) dt_s (C_t . B_s) x_s  +  D x_t
+//   S'   = exp(c_L) S  +  sum_s exp(c_L - c_s) dt_s B_s x_s^T
+// grid (sequence, head, P / 64): wave w owns the 16 state columns p0 + 16 w .. +15 (all N rows:
+// N / 16 accumulator tiles).  Per chunk a wave issues about 12 + 4 N / 16 ... MFMAs instead of
+// 16 x 2 N / 16 scalar FMA rounds per lane; tokens past the end of the last chunk get dt = a = 0,
+// so they neither decay nor feed the state.  Operand orders are permuted as in attn_sigmoid.hip so
+// that accumulators feed the next MFMA without shuffles.
+template <typename T, int NR>
+__global__ __launch_bounds__(256) void ssm_chunk_kernel(const T* __restrict__ xbc, long xs, const T* __restrict__ dtp,
+                                                        long dts, int heads, int P, int N, int groups,
+                                                        const float* __restrict__ dt_bias,
+                                                        const float* __restrict__ A_log, const float* __restrict__ Dp,
+                                                        float* __restrict__ state, const int* __restrict__ cu,
+                                                        const int* __restrict__ slots,
+                                                        const int* __restrict__ positions, float* __restrict__ y,
+                                                        long ys) {
+  constexpr int NP = NR * 16, LD = NP + 4, L = 16;
+  constexpr int EV = 16 / sizeof(T);
+  __shared__ __attribute__((aligned(16))) float sB[L][LD];
+  __shared__ __attribute__((aligned(16))) float sC[L][LD];
+  __shared__ float sx[L][64], sdt[L], sa[L], scum[L];
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, p0 = blockIdx.z * 64;
+  const int lane = tid & 63, w = tid >> 6, n16 = lane & 15, g = lane >> 4;
+  const int pcol = p0 + 16 * w + n16;
+  const bool pv = pcol < P;
+  const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
+  if (len <= 0) return;
+  if (slot < 0) {
+    for (int i = tid; i < len * 64; i += 256)
+      if (p0 + (i & 63) < P) y[(long)(row0 + (i >> 6)) * ys + (long)h * P + p0 + (i & 63)] = 0.f;
+    return;
+  }
+  const int inner = heads * P, grp = h / (heads / groups);
+  const long xo = (long)h * P + p0, bo = inner + (long)grp * N, co = inner + (long)groups * N + (long)grp * N;
+  float* sp = state + (((long)slot * heads + h) * P + (pv ? pcol : 0)) * N;
+  const bool past = positions[row0] > 0;
+  floatx4 S[NR];
+#pragma unroll
+  for (int nt = 0; nt < NR; ++nt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = nt * 16 + 4 * g + j;
+      S[nt][j] = (past && pv && n < N) ? sp[n] : 0.f;
+    }
+  const float nA = -expf(A_log[h]), db = dt_bias[h], Dh = Dp[h];
+  const bool vec = N % EV == 0 && xs % EV == 0 && bo % EV == 0 && co % EV == 0 &&
+                   (reinterpret_cast<uintptr_t>(xbc) & 15) == 0;
+  for (int t0 = 0; t0 < len; t0 += L) {
+    const int tl = min(L, len - t0);
+    __syncthreads();
+    if (vec) {
+      const int cpr = NP / EV, ncpr = N / EV;
+      for (int i = tid; i < L * cpr * 2; i += 256) {
+        const int which = i / (L * cpr), r = i % (L * cpr), t = r / cpr, c = r % cpr;
+        float* dst = (which ? sC[t] : sB[t]) + c * EV;
+        if (t < tl && c < ncpr) {
+          const T* src = xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + c * EV;
+          if constexpr (sizeof(T) == 2) {
+            const short8 v = *reinterpret_cast<const short8*>(src);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dst[e] = bf2f((bf16_t)v[e]);
+          } else {
+            *reinterpret_cast<floatx4*>(dst) = *reinterpret_cast<const floatx4*>(src);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < EV; ++e) dst[e] = 0.f;
+        }
+      }
+    } else {
+      for (int i = tid; i < L * NP * 2; i += 256) {
+        const int which = i / (L * NP), r = i % (L * NP), t = r / NP, n = r % NP;
+        (which ? sC[t] : sB[t])[n] =
+            (t < tl && n < N) ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + n) : 0.f;
+      }
+    }
+    for (int i = tid; i < L * 64; i += 256) {
+      const int t = i >> 6, c = i & 63;
+      sx[t][c] = (t < tl && p0 + c < P) ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + xo + c) : 0.f;
+    }
+    if (tid < L) {
+      float dt = 0.f;
+      if (tid < tl) {
+        const float a = ldf<T>(dtp + (long)(row0 + t0 + tid) * dts + h) + db;
+        dt = a > 20.f ? a : log1pf(expf(a));
+      }
+      sdt[tid] = dt;
+      sa[tid] = nA * dt;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      float c = 0.f;
+#pragma unroll
+      for (int t = 0; t < L; ++t) {
+        c += sa[t];
+        scum[t] = c;
+      }
+    }
+    __syncthreads();
+    // G^T: lane (t = n16, g) gets G[t][s = 4g + j] = C_t . B_s
+    floatx4 gt = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int nb = 0; nb < NR; ++nb) {
+      const floatx4 a4 = *reinterpret_cast<const floatx4*>(&sB[n16][nb * 16 + 4 * g]);
+      const floatx4 b4 = *reinterpret_cast<const floatx4*>(&sC[n16][nb * 16 + 4 * g]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gt = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], b4[j], gt, 0, 0, 0);
+    }
+    const float ct = scum[n16], cl = scum[L - 1];
+    float M[4], xv[4], wv[4], ec[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int sj = 4 * g + j;
+      const float cs = scum[sj], ds = sdt[sj];
+      M[j] = sj <= n16 ? gt[j] * expf(ct - cs) * ds : 0.f;
+      xv[j] = sx[sj][16 * w + n16];
+      wv[j] = expf(cl - cs) * ds;
+      ec[j] = expf(cs);
+    }
+    // y: rows t = 4g + j, column p = n16 of this wave's tile
+    floatx4 ya = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int nt = 0; nt < NR; ++nt) {
+      const floatx4 c4 = *reinterpret_cast<const floatx4*>(&sC[n16][nt * 16 + 4 * g]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ya = __builtin_amdgcn_mfma_f32_16x16x4f32(c4[j], S[nt][j], ya, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ya[j] *= ec[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ya = __builtin_amdgcn_mfma_f32_16x16x4f32(M[j], xv[j], ya, 0, 0, 0);
+    if (pv) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int t = 4 * g + j;
+        if (t < tl) y[(long)(row0 + t0 + t) * ys + (long)h * P + pcol] = ya[j] + Dh * xv[j];
+      }
+    }
+    // state: rows n = 16 nt + 4g + j, column p = n16
+    const float dec = expf(cl);
+#pragma unroll
+    for (int nt = 0; nt < NR; ++nt) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) S[nt][j] *= dec;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        S[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sB[4 * g + j][nt * 16 + n16] * wv[j], xv[j], S[nt], 0, 0, 0);
+    }
+  }
+  if (pv) {
+#pragma unroll
+    for (int nt = 0; nt < NR; ++nt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = nt * 16 + 4 * g + j;
+        if (n < N) sp[n] = S[nt][j];
+      }
+  }
+}
+
 // grid (row, norm group): out = (y * silu(z)) / sqrt(mean_group((y silu z)^2) + eps) * w
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* __restrict__ y, long ys,
@@ -276,10 +440,28 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* _
   }
 }
 
+// prompt portions (some sequence of the step has >= kChunkMin rows): the chunked MFMA kernel
+constexpr int kChunkMin = 8;
+
 template <typename T>
 int scan_t(const T* xbc, long xs, const T* dtp, long dts, int S, int heads, int P, int N, int groups,
            const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
-           const int* positions, float* y, long ys, hipStream_t st) {
+           const int* positions, float* y, long ys, int max_len, hipStream_t st) {
+  if (max_len >= kChunkMin) {
+    dim3 cgrid(S, heads, (P + 63) / 64);
+#define LK_CHUNK(NR)                                                                                                   \
+  ssm_chunk_kernel<T, NR><<<cgrid, 256, 0, st>>>(xbc, xs, dtp, dts, heads, P, N, groups, dt_bias, A_log, D, state, cu, \
+                                                 slots, positions, y, ys)
+    if (N <= 16) LK_CHUNK(1);
+    else if (N <= 32) LK_CHUNK(2);
+    else if (N <= 64) LK_CHUNK(4);
+    else if (N <= 128) LK_CHUNK(8);
+    else if (N <= 256) LK_CHUNK(16);
+    else return -1;
+#undef LK_CHUNK
+    LK_CHECK_LAUNCH();
+    return 0;
+  }
   dim3 grid(S, heads, (P + 15) / 16);
 #define LK_SCAN(NR)                                                                                                 \
   ssm_scan_kernel<T, NR><<<grid, 256, 0, st>>>(xbc, xs, dtp, dts, heads, P, N, groups, dt_bias, A_log, D, state, cu, \
@@ -320,13 +502,13 @@ int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const 
 
 int lk_ssm_scan(const void* xbc, long xs, const void* dt, long dts, int S, int heads, int P, int N, int groups,
                 const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
-                const int* positions, float* y, long ys, int esz, hipStream_t st) {
+                const int* positions, float* y, long ys, int max_len, int esz, hipStream_t st) {
   if (S <= 0) return 0;
   if (heads <= 0 || groups <= 0 || heads % groups || P <= 0 || N <= 0) return -1;
   return esz == 2 ? scan_t<bf16_t>((const bf16_t*)xbc, xs, (const bf16_t*)dt, dts, S, heads, P, N, groups, dt_bias,
-                                   A_log, D, state, cu, slots, positions, y, ys, st)
+                                   A_log, D, state, cu, slots, positions, y, ys, max_len, st)
                   : scan_t<float>((const float*)xbc, xs, (const float*)dt, dts, S, heads, P, N, groups, dt_bias, A_log,
-                                  D, state, cu, slots, positions, y, ys, st);
+                                  D, state, cu, slots, positions, y, ys, max_len, st);
 }
 
 int lk_gated_group_rmsnorm(const float* y, long ys, const void* z, long zs, const float* w, long rows, int inner,

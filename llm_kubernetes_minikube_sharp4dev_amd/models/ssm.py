@@ -65,6 +65,6 @@ def mamba2_mixer(h, w_in, conv_w, conv_b, dt_bias, A_log, D, norm_w, w_out, spec
     xbc = ops.conv_silu(u, inner, C, conv_w, conv_b, conv_state, meta.seq_cu, meta.state_slots, meta.positions,
                         meta.max_seq_len)
     y = ops.ssm_scan(xbc, u[:, inner + C:inner + C + spec.heads], spec.heads, spec.vdim, spec.state, spec.groups, dt_bias, A_log, D,
-                     ssm_state, meta.seq_cu, meta.state_slots, meta.positions)
+                     ssm_state, meta.seq_cu, meta.state_slots, meta.positions, max_len=meta.max_seq_len)
     g = ops.gated_group_rmsnorm(y, u[:, :inner], norm_w, spec.norm_groups, eps)
     return ops.linear(g, w_out)

@@ -225,12 +225,15 @@ def conv_silu(u, col0: int, C: int, w, bias, state, cu, slots, positions, max_le
     return out
 
 
-def ssm_scan(xbc, dt, heads: int, P: int, N: int, groups: int, dt_bias, A_log, D, state, cu, slots, positions):
+def ssm_scan(xbc, dt, heads: int, P: int, N: int, groups: int, dt_bias, A_log, D, state, cu, slots, positions,
+             max_len: int = 1):
     """y f32 [T, heads * P]: per head, S_t = exp(-exp(A_log) dt_t) S_{t-1} + dt_t B_t x_t^T and
     y_t = S_t^T C_t + D x_t with dt_t = softplus(dt_t + dt_bias); x | B | C are the columns of
-    ``xbc``; the f32 state of each sequence is read from / left in ``state[slot]`` ([heads, P, N])."""
+    ``xbc``; the f32 state of each sequence is read from / left in ``state[slot]`` ([heads, P, N]).
+    ``max_len``: the longest sequence of the step (from 8 rows on the GPU runs the chunked matrix
+    form, below that the token-by-token kernel)."""
     if use_hip(xbc):
-        return lib().ssm_scan(xbc, dt, heads, P, N, groups, dt_bias, A_log, D, state, cu, slots, positions)
+        return lib().ssm_scan(xbc, dt, heads, P, N, groups, dt_bias, A_log, D, state, cu, slots, positions, int(max_len))
     inner = heads * P
     y = torch.zeros(xbc.shape[0], inner, dtype=torch.float32, device=xbc.device)
     cul, sl = cu.tolist(), slots.tolist()
