@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256) void ssm_chunk_kernel(const T* __restrict__ xb
   constexpr int EV = 16 / sizeof(T);
   __shared__ __attribute__((aligned(16))) float sB[L][LD];
   __shared__ __attribute__((aligned(16))) float sC[L][LD];
-  __shared__ float sx[L][64], sdt[L], sa[L], scum[L];
+  __shared__ float sx[L][64], sdt[L], sa[L];
   const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, p0 = blockIdx.z * 64;
   const int lane = tid & 63, w = tid >> 6, n16 = lane & 15, g = lane >> 4;
   const int pcol = p0 + 16 * w + n16;
@@ -305,58 +305,87 @@ __global__ __launch_bounds__(256) void ssm_chunk_kernel(const T* __restrict__ xb
   const float nA = -expf(A_log[h]), db = dt_bias[h], Dh = Dp[h];
   const bool vec = N % EV == 0 && xs % EV == 0 && bo % EV == 0 && co % EV == 0 &&
                    (reinterpret_cast<uintptr_t>(xbc) & 15) == 0;
+  // vector path: the next chunk's operands are requested before this chunk's products are issued
+  constexpr int NPF = (2 * L * NP / EV + 255) / 256;
+  uint4_t pre[NPF];
+  float prex[4], predt = 0.f;
+  auto fetch = [&](int t0) {
+    const int tl = min(L, len - t0), cpr = NP / EV, ncpr = N / EV;
+#pragma unroll
+    for (int k = 0; k < NPF; ++k) {
+      const int i = tid + 256 * k;
+      pre[k] = uint4_t{0u, 0u, 0u, 0u};
+      if (i < L * cpr * 2) {
+        const int which = i / (L * cpr), r = i % (L * cpr), t = r / cpr, c = r % cpr;
+        if (t < tl && c < ncpr)
+          pre[k] = *reinterpret_cast<const uint4_t*>(xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + c * EV);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = tid + 256 * k, t = i >> 6, c = i & 63;
+      prex[k] = (t < tl && p0 + c < P) ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + xo + c) : 0.f;
+    }
+    predt = tid < tl ? ldf<T>(dtp + (long)(row0 + t0 + tid) * dts + h) : 0.f;
+  };
+  if (vec) fetch(0);
   for (int t0 = 0; t0 < len; t0 += L) {
     const int tl = min(L, len - t0);
     __syncthreads();
+    float dtraw = 0.f;
     if (vec) {
-      const int cpr = NP / EV, ncpr = N / EV;
-      for (int i = tid; i < L * cpr * 2; i += 256) {
-        const int which = i / (L * cpr), r = i % (L * cpr), t = r / cpr, c = r % cpr;
-        float* dst = (which ? sC[t] : sB[t]) + c * EV;
-        if (t < tl && c < ncpr) {
-          const T* src = xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + c * EV;
+      const int cpr = NP / EV;
+#pragma unroll
+      for (int k = 0; k < NPF; ++k) {
+        const int i = tid + 256 * k;
+        if (i < L * cpr * 2) {
+          const int which = i / (L * cpr), r = i % (L * cpr), t = r / cpr, c = r % cpr;
+          float* dst = (which ? sC[t] : sB[t]) + c * EV;
           if constexpr (sizeof(T) == 2) {
-            const short8 v = *reinterpret_cast<const short8*>(src);
+            const short8 v = __builtin_bit_cast(short8, pre[k]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) dst[e] = bf2f((bf16_t)v[e]);
           } else {
-            *reinterpret_cast<floatx4*>(dst) = *reinterpret_cast<const floatx4*>(src);
+            *reinterpret_cast<uint4_t*>(dst) = pre[k];
           }
-        } else {
-#pragma unroll
-          for (int e = 0; e < EV; ++e) dst[e] = 0.f;
         }
       }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int i = tid + 256 * k;
+        sx[i >> 6][i & 63] = prex[k];
+      }
+      dtraw = predt;
     } else {
       for (int i = tid; i < L * NP * 2; i += 256) {
         const int which = i / (L * NP), r = i % (L * NP), t = r / NP, n = r % NP;
         (which ? sC[t] : sB[t])[n] =
             (t < tl && n < N) ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + (which ? co : bo) + n) : 0.f;
       }
-    }
-    for (int i = tid; i < L * 64; i += 256) {
-      const int t = i >> 6, c = i & 63;
-      sx[t][c] = (t < tl && p0 + c < P) ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + xo + c) : 0.f;
+      for (int i = tid; i < L * 64; i += 256) {
+        const int t = i >> 6, c = i & 63;
+        sx[t][c] = (t < tl && p0 + c < P) ? ldf<T>(xbc + (long)(row0 + t0 + t) * xs + xo + c) : 0.f;
+      }
+      if (tid < tl) dtraw = ldf<T>(dtp + (long)(row0 + t0 + tid) * dts + h);
     }
     if (tid < L) {
       float dt = 0.f;
       if (tid < tl) {
-        const float a = ldf<T>(dtp + (long)(row0 + t0 + tid) * dts + h) + db;
+        const float a = dtraw + db;
         dt = a > 20.f ? a : log1pf(expf(a));
       }
       sdt[tid] = dt;
       sa[tid] = nA * dt;
     }
     __syncthreads();
-    if (tid == 0) {
-      float c = 0.f;
+    if (vec && t0 + L < len) fetch(t0 + L);
+    // inclusive prefix of the log-decays inside every 16-lane group: lane n16 ends up with c_(n16)
+    float cum = sa[n16];
 #pragma unroll
-      for (int t = 0; t < L; ++t) {
-        c += sa[t];
-        scum[t] = c;
-      }
+    for (int o = 1; o < 16; o <<= 1) {
+      const float v = __shfl_up(cum, o, 16);
+      if (n16 >= o) cum += v;
     }
-    __syncthreads();
     // G^T: lane (t = n16, g) gets G[t][s = 4g + j] = C_t . B_s
     floatx4 gt = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -366,12 +395,12 @@ __global__ __launch_bounds__(256) void ssm_chunk_kernel(const T* __restrict__ xb
 #pragma unroll
       for (int j = 0; j < 4; ++j) gt = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], b4[j], gt, 0, 0, 0);
     }
-    const float ct = scum[n16], cl = scum[L - 1];
+    const float ct = cum, cl = __shfl(cum, 15, 16);
     float M[4], xv[4], wv[4], ec[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int sj = 4 * g + j;
-      const float cs = scum[sj], ds = sdt[sj];
+      const float cs = __shfl(cum, sj, 16), ds = sdt[sj];
       M[j] = sj <= n16 ? gt[j] * expf(ct - cs) * ds : 0.f;
       xv[j] = sx[sj][16 * w + n16];
       wv[j] = expf(cl - cs) * ds;
