@@ -311,7 +311,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void unitnorm_kv_write_kernel(T* __restrict__ qkv, long qs, int H, int G, int dim,
                                                                 int vdim, int norm_dim, float eps, T* __restrict__ kc,
                                                                 T* __restrict__ vc, const int* __restrict__ slots,
-                                                                int BS) {
+                                                                int BS, const T* __restrict__ bias) {
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int slot = slots[t];
@@ -321,24 +321,26 @@ __global__ __launch_bounds__(256) void unitnorm_kv_write_kernel(T* __restrict__ 
   for (int job = w; job < H + 2 * G; job += 4) {
     if (job < H + G) {  // a q or k head: x / sqrt(mean(x^2) + eps)
       T* x = row + (long)job * dim;
+      const T* bb = bias ? bias + (long)job * dim : nullptr;  // the projection's bias, added here in f32
       float ss = 0.f;
       for (int c = lane; c < dim; c += 64) {
-        const float v = El<T>::ld(x + c);
+        const float v = El<T>::ld(x + c) + (bb ? El<T>::ld(bb + c) : 0.f);
         ss += v * v;
       }
       ss = wave_sum(ss);
       const float inv = 1.f / sqrtf(ss / (float)norm_dim + eps);
       if (job < H) {
-        for (int c = lane; c < dim; c += 64) El<T>::st(x + c, El<T>::ld(x + c) * inv);
+        for (int c = lane; c < dim; c += 64) El<T>::st(x + c, (El<T>::ld(x + c) + (bb ? El<T>::ld(bb + c) : 0.f)) * inv);
       } else if (slot >= 0) {
         T* dst = kc + ((blk * G + (job - H)) * BS + off) * dim;
-        for (int c = lane; c < dim; c += 64) El<T>::st(dst + c, El<T>::ld(x + c) * inv);
+        for (int c = lane; c < dim; c += 64) El<T>::st(dst + c, (El<T>::ld(x + c) + (bb ? El<T>::ld(bb + c) : 0.f)) * inv);
       }
     } else if (slot >= 0) {  // a v head, filed key-contiguous
       const int gh = job - H - G;
       const T* x = row + (long)(H + G) * dim + (long)gh * vdim;
+      const T* bb = bias ? bias + (long)(H + G) * dim + (long)gh * vdim : nullptr;
       T* dst = vc + (blk * G + gh) * (long)vdim * BS + off;
-      for (int c = lane; c < vdim; c += 64) dst[(long)c * BS] = x[c];
+      for (int c = lane; c < vdim; c += 64) El<T>::st(dst + (long)c * BS, El<T>::ld(x + c) + (bb ? El<T>::ld(bb + c) : 0.f));
     }
   }
 }
@@ -413,15 +415,15 @@ SigParams make_params(const void* q, long qs, const void* kc, const void* vc, co
 int lk_sigattn_supported(int H, int G, int dim, int vdim, int BS, int esz) { return shape_ok(H, G, dim, vdim, BS, esz); }
 
 int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, int norm_dim, float eps, void* kc, void* vc,
-                         const int* slots, int BS, int esz, hipStream_t st) {
+                         const int* slots, int BS, const void* bias, int esz, hipStream_t st) {
   if (T <= 0) return 0;
   if (!shape_ok(H, G, dim, vdim, BS, esz) || norm_dim < 1 || norm_dim > dim) return -1;
   if (esz == 2)
     unitnorm_kv_write_kernel<bf16_t><<<(unsigned)T, 256, 0, st>>>((bf16_t*)qkv, qs, H, G, dim, vdim, norm_dim, eps, (bf16_t*)kc,
-                                                                  (bf16_t*)vc, slots, BS);
+                                                                  (bf16_t*)vc, slots, BS, (const bf16_t*)bias);
   else
     unitnorm_kv_write_kernel<float><<<(unsigned)T, 256, 0, st>>>((float*)qkv, qs, H, G, dim, vdim, norm_dim, eps, (float*)kc,
-                                                                 (float*)vc, slots, BS);
+                                                                 (float*)vc, slots, BS, (const float*)bias);
   LK_CHECK_LAUNCH();
   return 0;
 }

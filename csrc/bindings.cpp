@@ -1098,7 +1098,8 @@ std::vector<at::Tensor> embed_pos(const at::Tensor& ids, const at::Tensor& posit
   return keep_copy ? std::vector<at::Tensor>{x, copy} : std::vector<at::Tensor>{x};
 }
 
-at::Tensor stream_rmsnorm(at::Tensor& x, const c10::optional<at::Tensor>& a, const c10::optional<at::Tensor>& b,
+at::Tensor stream_rmsnorm(at::Tensor& x, const c10::optional<at::Tensor>& a, const c10::optional<at::Tensor>& a_bias,
+                          const c10::optional<at::Tensor>& b,
                           const c10::optional<at::Tensor>& e, double mult, const c10::optional<at::Tensor>& w,
                           double woff, double eps, const c10::optional<at::Tensor>& idx, at::ScalarType out_dtype) {
   CHECK_CUDA(x); CHECK_F32(x); CHECK_CONTIG(x);
@@ -1112,7 +1113,7 @@ at::Tensor stream_rmsnorm(at::Tensor& x, const c10::optional<at::Tensor>& a, con
   if (b) { CHECK_CUDA(*b); same_type(*b, out, "b"); CHECK_LASTDIM(*b); TORCH_CHECK(b->dim() == 2 && b->size(0) == T && b->size(1) == W, "b shape"); bs = b->stride(0); }
   if (e) { CHECK_CUDA(*e); CHECK_F32(*e); CHECK_CONTIG(*e); TORCH_CHECK(e->sizes() == x.sizes(), "e shape"); }
   if (idx) { CHECK_CUDA(*idx); TORCH_CHECK(idx->scalar_type() == at::kLong && idx->is_contiguous(), "idx must be int64"); }
-  CHECK_RC(lk_stream_rmsnorm(x.data_ptr<float>(), a ? a->data_ptr() : nullptr, as, b ? b->data_ptr() : nullptr, bs,
+  CHECK_RC(lk_stream_rmsnorm(x.data_ptr<float>(), a ? a->data_ptr() : nullptr, as, fpo(a_bias, W, "a_bias"), b ? b->data_ptr() : nullptr, bs,
                              e ? e->data_ptr<float>() : nullptr, (float)mult, fpo(w, W, "w"), (float)woff, (float)eps,
                              idx ? idx->data_ptr<int64_t>() : nullptr, out.size(0), out.data_ptr(), out.stride(0), W, esz,
                              cur_stream()), "stream_rmsnorm");
@@ -1148,17 +1149,20 @@ void check_sig_caches(const at::Tensor& act, const at::Tensor& kc, const at::Ten
 }
 
 void unitnorm_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64_t vdim, int64_t norm_dim, double eps, at::Tensor& kc,
-                       at::Tensor& vc, const at::Tensor& slots) {
+                       at::Tensor& vc, const at::Tensor& slots, const c10::optional<at::Tensor>& bias) {
   CHECK_CUDA(qkv); CHECK_LASTDIM(qkv); CHECK_I32(slots); CHECK_CONTIG(slots);
   const int esz = esz_of(qkv, "qkv");
   TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) == (H + G) * dim + G * vdim, "qkv must be [T, (H + G) dim + G vdim]");
   TORCH_CHECK(slots.numel() >= qkv.size(0), "slots");
   check_sig_caches(qkv, kc, vc, G, dim, vdim);
   const int BS = kc.size(2);
-  const long nslots = kc.size(0) * BS;
-  (void)nslots;
+  if (bias) {
+    CHECK_CUDA(*bias); same_type(*bias, qkv, "bias");
+    TORCH_CHECK(bias->is_contiguous() && bias->numel() == qkv.size(1), "bias must be [(H + G) dim + G vdim]");
+  }
   CHECK_RC(lk_unitnorm_kv_write(qkv.data_ptr(), qkv.stride(0), qkv.size(0), H, G, dim, vdim, norm_dim, (float)eps, kc.data_ptr(),
-                                vc.data_ptr(), ip(slots), BS, esz, cur_stream()), "unitnorm_kv_write");
+                                vc.data_ptr(), ip(slots), BS, bias ? bias->data_ptr() : nullptr, esz, cur_stream()),
+           "unitnorm_kv_write");
 }
 
 at::Tensor sigattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt,

@@ -221,7 +221,7 @@ int lk_gather_rows(bf16_t* out, const bf16_t* x, long xs, const long* idx, long 
 int lk_embed_pos(const int* ids, const int* positions, const void* tok, int vocab, const void* pos, int max_pos, long rows,
                  int W, float* x, float* copy, int esz, hipStream_t st);
 int lk_stream_embed_errors();  // ids / positions outside their tables seen by lk_embed_pos (their rows are zero)
-int lk_stream_rmsnorm(float* x, const void* a, long as, const void* b, long bs, const float* e, float m, const float* w,
+int lk_stream_rmsnorm(float* x, const void* a, long as, const float* a_bias, const void* b, long bs, const float* e, float m, const float* w,
                       float woff, float eps, const long* idx, long out_rows, void* out, long os, int W, int esz,
                       hipStream_t st);
 int lk_silu_mul_f32(const float* x, long xs, float* out, long os, long rows, int I, hipStream_t st);
@@ -231,7 +231,7 @@ int lk_softcap(const void* in, long is, float cap, float* out, long os, long row
 // [NB, G, vdim, BS])
 int lk_sigattn_supported(int H, int G, int dim, int vdim, int BS, int esz);
 int lk_unitnorm_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, int norm_dim, float eps, void* kc, void* vc,
-                         const int* slots, int BS, int esz, hipStream_t st);
+                         const int* slots, int BS, const void* bias, int esz, hipStream_t st);
 int lk_sigattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride,
                        const int* cu_q, const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H,
                        int G, int dim, int vdim, int BS, float scale, const float* r1, const float* r2, const float* pb,

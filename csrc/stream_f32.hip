@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void embed_pos_kernel(const int* __restrict__ 
 
 template <typename T>
 __global__ __launch_bounds__(256) void stream_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ a, long as,
-                                                             const T* __restrict__ b, long bs,
+                                                             const float* __restrict__ ab, const T* __restrict__ b, long bs,
                                                              const float* __restrict__ e, float m,
                                                              const float* __restrict__ w, float woff, float eps,
                                                              const long* __restrict__ idx, T* __restrict__ out, long os,
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void stream_rmsnorm_kernel(float* __restrict__
   for (int c = threadIdx.x; c < W; c += 256) {
     float v = x[row * W + c];
     float d = 0.f;
-    if (a) d += ldv<T>(a + row * as + c);
+    if (a) d += ldv<T>(a + row * as + c) + (ab ? ab[c] : 0.f);
     if (b) d += ldv<T>(b + row * bs + c);
     v += m * d;
     if (e) v += e[row * W + c];
@@ -72,12 +72,71 @@ __global__ __launch_bounds__(256) void stream_rmsnorm_kernel(float* __restrict__
     } else {
       v = x[row * W + c];
       float d = 0.f;
-      if (a) d += ldv<T>(a + row * as + c);
+      if (a) d += ldv<T>(a + row * as + c) + (ab ? ab[c] : 0.f);
       if (b) d += ldv<T>(b + row * bs + c);
       v += m * d;
       if (e) v += e[row * W + c];
     }
     stv<T>(out + orow * os + c, v * inv * (w ? woff + w[c] : 1.f));
+  }
+}
+
+// The same with the row kept in registers and 16-byte (f32) / 8-byte (bf16) accesses: W % 4 == 0,
+// W <= 4 * 256 * MAXV, 16-byte aligned rows.  One read of every input, one write of x and of out.
+template <typename T, int MAXV>
+__global__ __launch_bounds__(256) void stream_rmsnorm_vec_kernel(float* __restrict__ x, const T* __restrict__ a, long as,
+                                                                 const float* __restrict__ ab, const T* __restrict__ b,
+                                                                 long bs,
+                                                                 const float* __restrict__ e, float m,
+                                                                 const float* __restrict__ w, float woff, float eps,
+                                                                 const long* __restrict__ idx, T* __restrict__ out,
+                                                                 long os, int W) {
+  __shared__ float red[4];
+  const long orow = blockIdx.x, row = idx ? idx[orow] : orow;
+  const int nv = W >> 2;
+  floatx4 v[MAXV];
+  float ss = 0.f;
+  auto ld4 = [](const T* p) -> floatx4 {
+    if constexpr (sizeof(T) == 2) {
+      const short4_t r = *reinterpret_cast<const short4_t*>(p);
+      return floatx4{bf2f((bf16_t)r[0]), bf2f((bf16_t)r[1]), bf2f((bf16_t)r[2]), bf2f((bf16_t)r[3])};
+    } else {
+      return *reinterpret_cast<const floatx4*>(p);
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      floatx4 t = *reinterpret_cast<const floatx4*>(x + row * W + 4 * c);
+      floatx4 d = {0.f, 0.f, 0.f, 0.f};
+      if (a) d += ld4(a + row * as + 4 * c);
+      if (a && ab) d += *reinterpret_cast<const floatx4*>(ab + 4 * c);
+      if (b) d += ld4(b + row * bs + 4 * c);
+      t += m * d;
+      if (e) t += *reinterpret_cast<const floatx4*>(e + row * W + 4 * c);
+      if (!idx && (a || b || e)) *reinterpret_cast<floatx4*>(x + row * W + 4 * c) = t;
+      v[i] = t;
+      ss += t[0] * t[0] + t[1] * t[1] + t[2] * t[2] + t[3] * t[3];
+    }
+  }
+  ss = block_sum<4>(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      floatx4 g = {1.f, 1.f, 1.f, 1.f};
+      if (w) g = *reinterpret_cast<const floatx4*>(w + 4 * c) + woff;
+      const floatx4 r = v[i] * inv * g;
+      T* o = out + orow * os + 4 * c;
+      if constexpr (sizeof(T) == 2) {
+        short4_t q = {(short)f2bf(r[0]), (short)f2bf(r[1]), (short)f2bf(r[2]), (short)f2bf(r[3])};
+        *reinterpret_cast<short4_t*>(o) = q;
+      } else {
+        *reinterpret_cast<floatx4*>(o) = r;
+      }
+    }
   }
 }
 
@@ -129,15 +188,31 @@ int lk_embed_pos(const int* ids, const int* positions, const void* tok, int voca
   return 0;
 }
 
-int lk_stream_rmsnorm(float* x, const void* a, long as, const void* b, long bs, const float* e, float m, const float* w,
+int lk_stream_rmsnorm(float* x, const void* a, long as, const float* a_bias, const void* b, long bs, const float* e, float m, const float* w,
                       float woff, float eps, const long* idx, long out_rows, void* out, long os, int W, int esz,
                       hipStream_t st) {
   if (out_rows <= 0) return 0;
+  const auto al = [](const void* p, long stride_bytes, int vec_bytes) {
+    return p == nullptr || (reinterpret_cast<uintptr_t>(p) % vec_bytes == 0 && stride_bytes % vec_bytes == 0);
+  };
+  constexpr int kMaxV = 8;
+  const int tv = esz == 2 ? 8 : 16;  // bytes of a 4-element access to the activations
+  if (W % 4 == 0 && W <= 4 * 256 * kMaxV && al(x, (long)W * 4, 16) && al(e, (long)W * 4, 16) && al(w, 0, 16) && al(a_bias, 0, 16) &&
+      al(a, as * (long)esz, tv) && al(b, bs * (long)esz, tv) && al(out, os * (long)esz, tv)) {
+    if (esz == 2)
+      stream_rmsnorm_vec_kernel<bf16_t, kMaxV><<<(unsigned)out_rows, 256, 0, st>>>(
+          x, (const bf16_t*)a, as, a_bias, (const bf16_t*)b, bs, e, m, w, woff, eps, idx, (bf16_t*)out, os, W);
+    else
+      stream_rmsnorm_vec_kernel<float, kMaxV><<<(unsigned)out_rows, 256, 0, st>>>(
+          x, (const float*)a, as, a_bias, (const float*)b, bs, e, m, w, woff, eps, idx, (float*)out, os, W);
+    LK_CHECK_LAUNCH();
+    return 0;
+  }
   if (esz == 2)
-    stream_rmsnorm_kernel<bf16_t><<<(unsigned)out_rows, 256, 0, st>>>(x, (const bf16_t*)a, as, (const bf16_t*)b, bs, e, m, w,
+    stream_rmsnorm_kernel<bf16_t><<<(unsigned)out_rows, 256, 0, st>>>(x, (const bf16_t*)a, as, a_bias, (const bf16_t*)b, bs, e, m, w,
                                                                       woff, eps, idx, (bf16_t*)out, os, W);
   else
-    stream_rmsnorm_kernel<float><<<(unsigned)out_rows, 256, 0, st>>>(x, (const float*)a, as, (const float*)b, bs, e, m, w,
+    stream_rmsnorm_kernel<float><<<(unsigned)out_rows, 256, 0, st>>>(x, (const float*)a, as, a_bias, (const float*)b, bs, e, m, w,
                                                                      woff, eps, idx, (float*)out, os, W);
   LK_CHECK_LAUNCH();
   return 0;

@@ -201,8 +201,9 @@ class SigmoidAttnSpec:
 
 
 def sigmoid_paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta, spec: SigmoidAttnSpec, r1, r2, pb,
-                            eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """qkv [T, (H + G) dim + G vdim] straight from the projection: unit-RMS q / k, k / v filed in
+                            eps: float, out: Optional[torch.Tensor] = None, qkv_bias=None) -> torch.Tensor:
+    """qkv [T, (H + G) dim + G vdim] straight from the projection (``qkv_bias``: its bias, if the
+    projection ran without it -- added in f32 by the norm kernel): unit-RMS q / k, k / v filed in
     the paged cache at ``meta.slots``, then prompt rows on the tiled prefill kernel and decode rows
     on the key-split decode kernel, both reading K / V from the cache (chunked prefill and decode
     are the same code path as whole prompts).  Returns [T, H vdim]."""
@@ -210,7 +211,8 @@ def sigmoid_paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta,
     T = qkv.shape[0]
     if out is None:
         out = torch.empty(T, H * vdim, dtype=qkv.dtype, device=qkv.device)
-    ops.unitnorm_kv_write(qkv, H, G, dim, vdim, eps, k_cache, v_cache, meta.slots, norm_dim=spec.norm_dim or dim)
+    ops.unitnorm_kv_write(qkv, H, G, dim, vdim, eps, k_cache, v_cache, meta.slots, norm_dim=spec.norm_dim or dim,
+                          bias=qkv_bias)
     Tp, Bd = meta.num_prefill_tokens, meta.num_decode
     if Tp:
         if meta.sig_tiles is None and qkv.is_cuda:

@@ -39,6 +39,11 @@ from .configs import LebepelConfig, pad_vocab
 from .ssm import Mamba2Spec, mamba2_mixer
 
 
+# The q|k|v bias either rides in the projection GEMM's epilogue (False) or is added in f32 by the
+# unit-norm kernel, so that the projection runs on the bias-free decode GEMMs (True).
+FUSE_QKV_BIAS = True
+
+
 class LebepelLayer(nn.Module):
     def __init__(self, cfg: LebepelConfig, spec, dtype, device):
         super().__init__()
@@ -56,7 +61,7 @@ class LebepelLayer(nn.Module):
             # head sizes padded to the kernels' 8-element fragments with zero weight rows / columns
             a = self.spec = SigmoidAttnSpec(t.heads, t.kv_heads, -(-t.dim // 8) * 8, -(-t.vdim // 8) * 8, t.scale, t.dim)
             self.qkv, self.qkv_b = P(a.qkv_out, W, **e), P(a.qkv_out, **e)
-            self.o, self.o_b = P(W, a.heads * a.vdim, **e), P(W, **e)
+            self.o, self.o_b = P(W, a.heads * a.vdim, **e), P(W, **f)   # o_b is added in the f32 stream update
             self.r1, self.r2, self.pb = P(a.heads, **f), P(a.heads, **f), P(a.heads, **f)
         else:
             s = self.spec = Mamba2Spec.from_dict(spec.mixer)
@@ -250,7 +255,7 @@ class LebepelModel(nn.Module):
             return []   # f32 activations run on the vendor library: nothing to route
         seen, out = set(), []
         for L in self.layers:
-            ws = [(L.in_proj, False), (L.o, False)] if L.type == "mamba2" else []
+            ws = [(L.in_proj, False), (L.o, False)] if L.type == "mamba2" else [(L.qkv, False), (L.o, False)]
             ws += [(L.gate_up, True), (L.down, False)] if L.ff else []
             for w, sw in ws:
                 if (tuple(w.shape), sw) not in seen:
@@ -290,12 +295,17 @@ class LebepelModel(nn.Module):
 
     # ------------------------------------------------------------------ forward
     def _mixer(self, L: LebepelLayer, h, meta: AttnMeta, cache):
+        """-> (mixer output without its output bias, that bias or None)."""
         if L.type == "attention":
-            qkv = ops.linear(h, L.qkv, L.qkv_b)
-            att = sigmoid_paged_attention(qkv, cache[0], cache[1], meta, L.spec, L.r1, L.r2, L.pb, self.cfg.norm_eps)
-            return ops.linear(att, L.o, L.o_b)
+            # the output projection runs bias-free (decode-sized steps then take the weight-streaming GEMMs):
+            # its bias is added by the stream update in f32; the q|k|v bias: see FUSE_QKV_BIAS
+            fuse = FUSE_QKV_BIAS
+            qkv = ops.linear(h, L.qkv) if fuse else ops.linear(h, L.qkv, L.qkv_b)
+            att = sigmoid_paged_attention(qkv, cache[0], cache[1], meta, L.spec, L.r1, L.r2, L.pb, self.cfg.norm_eps,
+                                          qkv_bias=L.qkv_b if fuse else None)
+            return ops.linear(att, L.o), L.o_b
         return mamba2_mixer(h, L.in_proj, L.conv_w, L.conv_b, L.dt_bias, L.A_log, L.D, L.mix_norm, L.o, L.spec,
-                            self.cfg.norm_eps, cache, meta)
+                            self.cfg.norm_eps, cache, meta), None
 
     def forward(self, ids: torch.Tensor, meta: AttnMeta, caches, taps: list = None) -> torch.Tensor:
         """-> normed hidden rows [R, W] that feed the LM head (``meta.logits_idx``, or every row).
@@ -304,18 +314,20 @@ class LebepelModel(nn.Module):
         cfg = self.cfg
         m, eps = cfg.residual_mult, cfg.norm_eps
         x, emb = ops.embed_pos(ids, meta.positions, self.embed, self.pos, keep_copy=self.reinject)
-        a = b = None
+        a = b = ab = None
         for run, (li, add_emb) in enumerate(self.runs):
             L = self.layers[li]
-            h = ops.stream_rmsnorm(x, a, b, emb if add_emb else None, m, L.norm1, 1.0, eps, out_dtype=self.dtype)
+            h = ops.stream_rmsnorm(x, a, b, emb if add_emb else None, m, L.norm1, 1.0, eps, out_dtype=self.dtype,
+                                   a_bias=ab)
             if taps is not None and run:  # the stream after the previous run, before this pass's re-injection
                 taps.append(x - emb if add_emb else x.clone())
-            a = self._mixer(L, h, meta, caches[run])
+            a, ab = self._mixer(L, h, meta, caches[run])
             b = ops.linear(ops.linear_swiglu_any(h, L.gate_up), L.down) if L.ff else None
         if taps is not None:
             d = a.float() if b is None else a.float() + b.float()
-            taps.append(x + m * d)
-        return ops.stream_rmsnorm(x, a, b, None, m, self.final_norm, 1.0, eps, idx=meta.logits_idx, out_dtype=self.dtype)
+            taps.append(x + m * (d if ab is None else d + ab))
+        return ops.stream_rmsnorm(x, a, b, None, m, self.final_norm, 1.0, eps, idx=meta.logits_idx, out_dtype=self.dtype,
+                                  a_bias=ab)
 
     def head(self, hidden):
         return ops.linear(hidden, self.lm_head)[:, : self.cfg.vocab_size]

@@ -40,12 +40,16 @@ def embed_pos(ids, positions, tok, pos, keep_copy: bool = False):
 
 
 def stream_rmsnorm(x, a=None, b=None, e=None, mult: float = 1.0, w=None, w_offset: float = 0.0, eps: float = 1e-5,
-                   idx=None, out_dtype=torch.bfloat16):
-    """``x += mult * (a + b) + e`` in place (f32), then ``x / sqrt(mean(x^2) + eps) * (w_offset + w)``
-    in ``out_dtype``.  With ``idx`` (int64 rows) only those rows are computed and ``x`` is left
-    as it was."""
+                   idx=None, out_dtype=torch.bfloat16, a_bias=None):
+    """``x += mult * (a + a_bias + b) + e`` in place (f32), then ``x / sqrt(mean(x^2) + eps) *
+    (w_offset + w)`` in ``out_dtype``.  With ``idx`` (int64 rows) only those rows are computed and
+    ``x`` is left as it was.  ``a_bias`` (f32 [W]): the bias of the projection that produced ``a``,
+    added here so that the projection itself runs on the bias-free GEMM kernels."""
     if use_hip(x):
-        return lib().stream_rmsnorm(x, a, b, e, float(mult), w, float(w_offset), float(eps), idx, out_dtype)
+        return lib().stream_rmsnorm(x, a, a_bias if a is not None else None, b, e, float(mult), w, float(w_offset),
+                                    float(eps), idx, out_dtype)
+    if a is not None and a_bias is not None:
+        a = a.float() + a_bias
     v = x if idx is None else x.index_select(0, idx)
     sel = (lambda t: t) if idx is None else (lambda t: t.index_select(0, idx))
     d = None
@@ -90,15 +94,18 @@ def sigattn_supported(H: int, G: int, dim: int, vdim: int, block_size: int, dtyp
 
 
 def unitnorm_kv_write(qkv, H: int, G: int, dim: int, vdim: int, eps: float, k_cache, v_cache, slots,
-                      norm_dim: Optional[int] = None):
+                      norm_dim: Optional[int] = None, bias=None):
     """Rows ``[q: H dim | k: G dim | v: G vdim]``: q and k become x / sqrt(mean(x^2) + eps) per head
     (f32 arithmetic; q in place, k into the cache), v goes into the cache.  Slots < 0 cache nothing.
-    ``norm_dim``: the divisor of the mean when the heads carry zero padding columns (default dim)."""
+    ``norm_dim``: the divisor of the mean when the heads carry zero padding columns (default dim).
+    ``bias`` [row width]: the projection's bias, added first in f32 (the projection then runs bias-free)."""
     norm_dim = dim if norm_dim is None else int(norm_dim)
     if use_hip(qkv):
-        lib().unitnorm_kv_write(qkv, H, G, dim, vdim, norm_dim, float(eps), k_cache, v_cache, slots)
+        lib().unitnorm_kv_write(qkv, H, G, dim, vdim, norm_dim, float(eps), k_cache, v_cache, slots, bias)
         return qkv
     T = qkv.shape[0]
+    if bias is not None:
+        qkv.copy_((qkv.float() + bias.float()).to(qkv.dtype))
     qk = qkv[:, : (H + G) * dim].float().view(T, H + G, dim)
     qk = qk / torch.sqrt(qk.pow(2).sum(-1, keepdim=True) / norm_dim + eps)
     qkv[:, : (H + G) * dim] = qk.reshape(T, -1).to(qkv.dtype)

@@ -37,9 +37,10 @@ def q16(t):
 
 # ---------------------------------------------------------------------------- residual stream
 @pytest.mark.parametrize("device,dtype", ALL)
-def test_embed_stream_norm_softcap(device, dtype):
+@pytest.mark.parametrize("W", [72, 70, 2052])   # vector path, scalar path, a row longer than one pass of the block
+def test_embed_stream_norm_softcap(W, device, dtype):
     g = torch.Generator().manual_seed(1)
-    V, P, W, T = 50, 40, 72, 9
+    V, P, T = 50, 40, 9
     tok, pos = q16(rnd(g, V, W)), q16(rnd(g, P, W))
     ids = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
     ps = torch.randint(0, P, (T,), generator=g, dtype=torch.int32)
@@ -48,11 +49,12 @@ def test_embed_stream_norm_softcap(device, dtype):
     assert x.dtype == torch.float32 and rel_err(x, want) < 1e-6 and torch.equal(x, e) and x.data_ptr() != e.data_ptr()
     a, b, w = q16(rnd(g, T, W)), q16(rnd(g, T, W)), q16(rnd(g, W, scale=0.1))
     eps, m = 1e-3, 0.37
-    xs = want + m * (a + b) + want
+    ab = q16(rnd(g, W, scale=0.3))
+    xs = want + m * (a + ab + b) + want
     hw = O.offset_rmsnorm(xs, w, eps)
     x0 = x.clone()
     h = ops.stream_rmsnorm(x, a.to(dtype).to(device), b.to(dtype).to(device), e, m, w.float().to(device), 1.0, eps,
-                           out_dtype=dtype)
+                           out_dtype=dtype, a_bias=ab.float().to(device))
     assert rel_err(x, xs) < 1e-6 and rel_err(h, hw) < tol(dtype) / 4
     # one input only, no weight offset, rows picked by index: the stream is left alone
     idx = torch.tensor([7, 0, 3], device=device)
@@ -142,8 +144,12 @@ def run_attention(spec, w, hs, schedule, bs, device, dtype, eps=1e-5):
     for chunks, decodes in schedule:
         meta = cache.meta(chunks, decodes)
         rows = [hs[s][st:st + n] for s, st, n in chunks] + [hs[s][p:p + 1] for s, p in decodes]
-        qkv = ops.linear(dev(torch.cat(rows)), wqkv, bqkv)
-        att = sigmoid_paged_attention(qkv, cache.kc, cache.vc, meta, spec, r1, r2, pb, eps)
+        if len(chunks) % 2:   # the bias inside the projection, or left to the norm kernel
+            qkv = ops.linear(dev(torch.cat(rows)), wqkv, bqkv)
+            att = sigmoid_paged_attention(qkv, cache.kc, cache.vc, meta, spec, r1, r2, pb, eps)
+        else:
+            qkv = ops.linear(dev(torch.cat(rows)), wqkv)
+            att = sigmoid_paged_attention(qkv, cache.kc, cache.vc, meta, spec, r1, r2, pb, eps, qkv_bias=bqkv)
         y = ops.linear(att, wo, bo).double().cpu()
         r = 0
         for s, st, n in list(chunks) + [(s, p, 1) for s, p in decodes]:
