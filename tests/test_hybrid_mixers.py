@@ -297,7 +297,8 @@ def oracle_mamba(spec, w, h, eps=1e-5):
 
 
 MSPECS = [Mamba2Spec(4, 16, 16, 2, 4, 2), Mamba2Spec(3, 8, 24, 1, 2, 1), Mamba2Spec(2, 40, 72, 2, 3, 4),
-          Mamba2Spec(6, 4, 8, 6, 1, 3)]
+          Mamba2Spec(6, 4, 8, 6, 1, 3), Mamba2Spec(1, 80, 136, 1, 4, 1), Mamba2Spec(2, 16, 32, 1, 5, 2),
+          Mamba2Spec(3, 6, 10, 3, 4, 1)]
 
 
 @pytest.mark.parametrize("device,dtype", ALL)
