@@ -249,7 +249,7 @@ class LLMEngine:
                     for k, (seq, _) in enumerate(rows):
                         at.setdefault(id(seq), []).append(k)
                     order = [k for seq, _, _ in items for k in at.get(id(seq), [])]
-                    lg = lg.float()
+                    lg = lg.to(torch.float32, copy=True)  # a captured step's logits live in the graph's static buffer
                     out = lg if order == list(range(len(order))) else lg.index_select(
                         0, torch.tensor(order, dtype=torch.long, device=lg.device))
             for rid in end:

@@ -51,6 +51,9 @@ CONFIGS = {
                        mult=0.4, cap=30.0),
     # sizes that are multiples of nothing convenient
     "odd": config([ff(ssm(3, 10, 12, 1, 3, 1), 50), ff(att(3, 1, 20, 12, 0.3), 50)], 36, vocab=61, loop=(1, 2, 2)),
+    # projections the MFMA / weight-streaming kernels tile: no vendor GEMM, decode steps captured in hipGraphs
+    "mid": config([ff(att(4, 2, 64, 64, 0.125), 512), ff(ssm(8, 32, 64, 2, 4, 2), 512)], 256, vocab=512, loop=(0, 2, 2),
+                  mult=0.5, cap=25.0),
 }
 _models = {}
 
@@ -257,3 +260,32 @@ def test_checkpoint_directory_selects_the_model_and_replays(tmp_path):
     bad["l0.mix.in"] = bad["l0.mix.in"][:-1]
     with pytest.raises(ValueError):
         LebepelModel(m2.cfg, dtype=torch.float32).load_state_dict_native(bad)
+
+
+@pytest.mark.gpu
+def test_captured_decode_graph_matches_the_oracle():
+    """bf16 on the GPU with sizes the framework's own GEMM kernels tile: decode steps replay a captured
+    hipGraph (state slots and block tables in its static buffers); prompt portions, then 40 single
+    tokens for two requests that start at different times, against the float64 forward."""
+    m, sd = model_and_weights("mid", "cuda", torch.bfloat16)
+    V = m.cfg.vocab_size
+    a, b = toks(90, V, 60), toks(75, V, 61)
+    wa, wb = O.forward(CONFIGS["mid"], sd, a), O.forward(CONFIGS["mid"], sd, b)
+    eng = engine(m, tokens=192, seqs=2)
+    ga = [eng.replay_step([("a", a[:33], list(range(33)))]), eng.replay_step([("a", a[33:50], list(range(17)))])]
+    gb = []
+    for i in range(40):
+        entries = [("a", [a[50 + i]], [0])]
+        if i == 5:
+            entries.append(("b", b[:35], list(range(35))))
+        elif i > 5:
+            entries.append(("b", [b[35 + i - 6]], [0]))
+        lg = eng.replay_step(entries)
+        ga.append(lg[:1])
+        if i >= 5:
+            gb.append(lg[1:])
+    captured = [k for k, st in eng.runner.graphs.items() if st.get("graph") is not None]
+    assert captured, "no decode bucket was captured"
+    for got, want, n in ((ga, wa, 90), (gb, wb, 35 + 34)):
+        ok, err = close(torch.cat(got), want[:n], torch.bfloat16)
+        assert ok, err
