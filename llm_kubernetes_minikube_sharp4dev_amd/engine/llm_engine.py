@@ -399,6 +399,7 @@ class LLMEngine:
 
         with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
             bad = int(ops.lib().embed_errors())  # this engine's device's counter
+            bad += max(0, int(ops.lib().stream_embed_errors()))  # the f32-stream embedding (ids or positions)
         if bad:
             raise RuntimeError(f"embedding: {bad} token id(s) outside the vocabulary were looked up (a tokenizer / "
                                f"model vocab mismatch); their rows were zero")

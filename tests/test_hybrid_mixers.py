@@ -196,13 +196,14 @@ def test_sigmoid_attention_whole_chunked_decoded(spec, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", ALL)
-def test_sigmoid_attention_one_far_key_stands_out(device, dtype):
+@pytest.mark.parametrize("far", [5, 15, 16, 32, 63])   # inside a page, a page's last and first slot, 32-key step edges
+def test_sigmoid_attention_one_far_key_stands_out(far, device, dtype):
     """Every weight is pushed to ~0 by a large negative head bias except where one query and one
     key are aligned and scaled up: the output row must be that key's value, through a context of
-    hundreds of keys and several pages, in a prompt portion and in a decode row; moving the key
-   , and a query that sits BEFORE the key sees nothing."""
+    hundreds of keys and several pages, in a prompt portion and in a decode row, and a query
+    that sits BEFORE the key sees nothing."""
     spec = SigmoidAttnSpec(2, 1, 16, 16, 1.0)
-    T, bs, far = 300, 16, 5
+    T, bs = 300, 16
     cache = PagedSeqs(spec, [T], bs, device, dtype)
     g = torch.Generator().manual_seed(5)
     k = rnd(g, T, 16, scale=0.05)

@@ -101,7 +101,6 @@ def test_whole_prompt_streams_and_logits(name, device, dtype):
     streams = []
     want = O.forward(CONFIGS[name], sd, t, streams)
     eng = engine(m)
-    seq_items = None
     # the f32 stream after every layer run, through the runner's own step inputs
     from llm_kubernetes_minikube_sharp4dev_amd.engine.sequence import Sequence
     sq = Sequence(list(t), SamplingParams(max_tokens=1))
