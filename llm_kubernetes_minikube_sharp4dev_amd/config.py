@@ -125,6 +125,8 @@ class ModelPresets:
         "llama3:70b": "llama-3-70b",
         "opt-125m": "opt-125m",
         "llama-tiny": "llama-tiny",
+        "lebepel-tiny": "lebepel-tiny",
+        "lebepel-1b": "lebepel-1b",
     })
     embedders: dict = field(default_factory=lambda: {
         "nomic-embed-text": "nomic-embed-text",
