@@ -35,7 +35,9 @@ def build_engine(model_dir: str, dtype: str = "bfloat16", max_tokens: int = 8192
         torch.backends.cudnn.allow_tf32 = False
     model = load_decoder_dir(model_dir, device=device, dtype=dt)
     num_blocks = max(1, -(-int(max_tokens) // block_size))
-    return LLMEngine(model, None, block_size=block_size, max_model_len=model.cfg.max_position, max_num_seqs=max_seqs,
+    # no request can be longer than the pool; a design without learned positions names no smaller bound
+    max_len = min(int(model.cfg.max_position), num_blocks * block_size)
+    return LLMEngine(model, None, block_size=block_size, max_model_len=max_len, max_num_seqs=max_seqs,
                      num_blocks=num_blocks, eos_ids=set(), use_graphs=use_graphs, enable_prefix_caching=True)
 
 

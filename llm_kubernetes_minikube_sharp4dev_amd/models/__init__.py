@@ -8,14 +8,19 @@ import torch
 
 from ..parallel.tp import SINGLE, TPGroup
 from .bert import EncoderModel
-from .configs import DECODERS, ENCODERS, DecoderConfig, EncoderConfig, LebepelConfig, decoder_config, encoder_config
+from .configs import (DECODERS, ENCODERS, DecoderConfig, EncoderConfig, LebepelConfig, PemidraConfig, decoder_config,
+                      encoder_config)
 from . import llama
 from .lebepel import LebepelModel
 from .llama import LlamaModel
 from .opt import OPTModel
+from .pemidra import PemidraModel, ranks_from_state_dict
 
 # decoder architectures by ``cfg.arch``
-DECODER_CLASSES = {"llama": LlamaModel, "opt": OPTModel, "lebepel": LebepelModel}
+DECODER_CLASSES = {"llama": LlamaModel, "opt": OPTModel, "lebepel": LebepelModel, "pemidra": PemidraModel}
+# designs with a checkpoint format of their own (config.json read by ``<Config>.from_json``, tensors by
+# ``load_state_dict_native``)
+NATIVE_CONFIGS = {"lebepel": LebepelConfig, "pemidra": PemidraConfig}
 
 
 def _load_safetensors_dir(path: str) -> dict:
@@ -31,11 +36,14 @@ def _load_safetensors_dir(path: str) -> dict:
 
 def build_decoder(name: str | DecoderConfig, device="cpu", dtype=torch.bfloat16, tp: TPGroup = SINGLE,
                   seed: int = 0, checkpoint: Optional[str] = None, **overrides):
-    cfg = name if isinstance(name, (DecoderConfig, LebepelConfig)) else decoder_config(name, **overrides)
+    cfg = name if isinstance(name, (DecoderConfig, LebepelConfig, PemidraConfig)) else decoder_config(name, **overrides)
     cls = DECODER_CLASSES[cfg.arch]
+    sd = _load_safetensors_dir(checkpoint) if checkpoint and cfg.arch in NATIVE_CONFIGS else None
+    if sd is not None and cfg.arch == "pemidra":
+        cfg = ranks_from_state_dict(cfg, sd)   # sizes that only the tensors' shapes give
     m = cls(cfg, tp, dtype, device)
-    if checkpoint and cfg.arch == "lebepel":
-        m.load_state_dict_native(_load_safetensors_dir(checkpoint))
+    if sd is not None:
+        m.load_state_dict_native(sd)
     elif checkpoint:
         m.load_hf_state_dict(_load_safetensors_dir(checkpoint))  # folds on the GPU itself
     else:
@@ -57,8 +65,8 @@ def checkpoint_architecture(path: str) -> Optional[str]:
     names = [str(d.get("architecture", ""))] + [str(a) for a in d.get("architectures", [])] + [str(d.get("model_type", ""))]
     for n in names:
         n = n.lower()
-        if n == "lebepel":
-            return "lebepel"
+        if n in NATIVE_CONFIGS:
+            return n
         if n.startswith("llama"):
             return "llama"
         if n.startswith("opt"):
@@ -75,8 +83,8 @@ def load_decoder_dir(path: str, device="cpu", dtype=torch.bfloat16, tp: TPGroup 
     if arch is None:
         raise ValueError(f"{path}: config.json names no decoder architecture of this framework")
     d = json.loads((Path(path) / "config.json").read_text())
-    if arch == "lebepel":
-        cfg = LebepelConfig.from_json(d, Path(path).name)
+    if arch in NATIVE_CONFIGS:
+        cfg = NATIVE_CONFIGS[arch].from_json(d, Path(path).name)
     elif arch == "llama":
         heads = d["num_attention_heads"]
         cfg = DecoderConfig(Path(path).name, "llama", d["num_hidden_layers"], d["hidden_size"], heads,
@@ -109,5 +117,5 @@ def build_encoder(name: str | EncoderConfig, device="cpu", dtype=torch.bfloat16,
 
 
 __all__ = ["build_decoder", "build_encoder", "load_decoder_dir", "checkpoint_architecture", "DECODER_CLASSES",
-           "LebepelConfig", "LebepelModel", "DECODERS", "ENCODERS", "DecoderConfig", "EncoderConfig",
+           "LebepelConfig", "LebepelModel", "PemidraConfig", "PemidraModel", "NATIVE_CONFIGS", "DECODERS", "ENCODERS", "DecoderConfig", "EncoderConfig",
            "LlamaModel", "OPTModel", "EncoderModel"]

@@ -228,6 +228,95 @@ def sigmoid_paged_attention(qkv: torch.Tensor, k_cache, v_cache, meta: AttnMeta,
     return out
 
 
+@dataclass
+class SinkAttnSpec:
+    """Grouped-query softmax attention whose denominator carries one extra term of score 0 (a sink
+    without a value), restricted by a mask (``ops.mask_first_key``: causal, fixed chunks of positions, or a
+    sliding window); q and k RMS-normed per head with a weight shared by the heads, the first
+    ``rot_dims`` dimensions of each head rotated by position (pairs i, i + rot_dims / 2), values divided
+    by their RMS, one score multiplier and one sigmoid output gate per head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    mask_kind: int = 0
+    mask_size: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    sink: bool = True
+    v_unit: bool = True
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "SinkAttnSpec":
+        mask, rot = m.get("mask") or {}, m.get("rot") or {}
+        kind = ops.MASK_CHUNK if mask.get("size") else ops.MASK_CAUSAL
+        if mask.get("kind") == "window":
+            kind = ops.MASK_WINDOW
+        s = cls(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                float(m.get("scale", int(m["dim"]) ** -0.5)), kind, int(mask.get("size", 0)), int(rot.get("dims", 0)),
+                float(rot.get("base", 10000.0)))
+        if s.heads % s.kv_heads or s.rot_dims % 2 or s.rot_dims > s.dim or (kind != ops.MASK_CAUSAL and s.mask_size < 1):
+            raise ValueError(f"unsupported attention sizes {m}")
+        return s
+
+    @property
+    def qkv_out(self) -> int:
+        return (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
+
+    def inv_freq(self, device) -> torch.Tensor:
+        """f32 [rot_dims / 2]: base^(-2 i / rot_dims), rounded once from float64."""
+        half = self.rot_dims // 2
+        f = torch.pow(torch.tensor(float(self.rot_base), dtype=torch.float64),
+                      -2.0 * torch.arange(half, dtype=torch.float64) / max(self.rot_dims, 1))
+        return f.to(torch.float32).to(device)
+
+    def cache_shapes(self, num_blocks: int, block_size: int):
+        """K [NB, G, BS, dim] and V key-contiguous [NB, G, vdim, BS] (csrc/attn_sink.hip)."""
+        return ((num_blocks, self.kv_heads, block_size, self.dim), (num_blocks, self.kv_heads, self.vdim, block_size))
+
+    def bytes_per_token(self, dtype) -> int:
+        return self.kv_heads * (self.dim + self.vdim) * torch.tensor([], dtype=dtype).element_size()
+
+
+def sink_paged_attention(qkvg: torch.Tensor, k_cache, v_cache, meta: AttnMeta, spec: SinkAttnSpec, q_w, k_w, inv_freq, hscale,
+                         eps: float, gate_col: Optional[int] = None, out: Optional[torch.Tensor] = None, norm_dim: int = 0,
+                         norm_vdim: int = 0) -> torch.Tensor:
+    """qkvg [T, q | k | v | ... gates] straight from the fused projection: q / k norm + rotation, value
+    norm and the paged K / V write in one kernel, then prompt rows on the tiled prefill kernel and decode
+    rows on the key-split decode kernel, both reading K / V from the cache (so portions of prompts and
+    decode rows are the same code path as whole prompts; the mask is taken from absolute positions).
+    ``gate_col``: column of the first head's raw output gate in ``qkvg``.  ``norm_dim`` / ``norm_vdim``: the
+    true head sizes (divisors of the RMS means) of a model whose heads carry zero padding columns up to
+    the kernels' vector width (0: dim / vdim).  Returns [T, H vdim]."""
+    H, G, dim, vdim = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    T = qkvg.shape[0]
+    if out is None:
+        out = torch.empty(T, H * vdim, dtype=qkvg.dtype, device=qkvg.device)
+    ops.normrope_kv_write(qkvg, H, G, dim, vdim, q_w, k_w, spec.rot_dims, inv_freq, meta.positions, eps, k_cache, v_cache,
+                          meta.slots, spec.v_unit, norm_dim or dim, norm_vdim or vdim)
+    gate = qkvg if gate_col is not None else None
+    gc = gate_col or 0
+    Tp, Bd = meta.num_prefill_tokens, meta.num_decode
+    if Tp:
+        if meta.sig_tiles is None and qkvg.is_cuda:
+            ts, tq = ops.sig_prefill_tiles(meta.q_lens_cpu, meta.ctx_lens_cpu)
+            meta.sig_tiles = (torch.from_numpy(ts).to(qkvg.device, non_blocking=True),
+                              torch.from_numpy(tq).to(qkvg.device, non_blocking=True))
+        ops.sink_attention_prefill(qkvg[:Tp], k_cache, v_cache, meta.block_tables_p, meta.cu_q, meta.ctx_lens_p, H, G, dim, vdim,
+                                   hscale, spec.mask_kind, spec.mask_size, spec.sink, gate[:Tp] if gate is not None else None, gc,
+                                   out[:Tp], tiles=meta.sig_tiles)
+    if Bd:
+        span = meta.block_tables_d.shape[1] * k_cache.shape[2]
+        if spec.mask_kind != ops.MASK_CAUSAL:
+            span = min(span, spec.mask_size)
+        Z = ops.sig_decode_splits(Bd, G, H // G, span)
+        ops.sink_attention_decode(qkvg[Tp:Tp + Bd], k_cache, v_cache, meta.block_tables_d, meta.ctx_lens_d, H, G, dim, vdim,
+                                  hscale, spec.mask_kind, spec.mask_size, spec.sink, gate[Tp:Tp + Bd] if gate is not None else None,
+                                  gc, out[Tp:Tp + Bd], splits=Z)
+    return out
+
+
 # ---------------------------------------------------------------- context parallelism
 def partial_attention(q, k, v, q_pos, k_pos0: int, scale: float, causal: bool = True):
     """Attention of q [S, Hq, D] over one key shard k/v [n, Hkv, D] whose key j sits at

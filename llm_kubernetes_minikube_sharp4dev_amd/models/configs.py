@@ -135,6 +135,74 @@ class LebepelConfig:
         return d
 
 
+@dataclass
+class PemidraConfig:
+    """The Pemidra design: post-norm layers over an f32 stream -- ``x <- LN(alpha x + ls * sub(x))`` for the
+    mixer and (where present) the gated tanh-GELU feed-forward -- with three kinds of mixer in any order:
+    ``retention`` (decayed linear attention), ``general_delta`` (generalized delta rule) and ``parallel``
+    (chunk-masked softmax attention with a sink beside a gated delta rule, their RMS-normed results
+    averaged).  No learned positions (rotary inside the attention only) and no cap on the logits.
+    Every size and constant comes from the checkpoint's ``config.json`` (:meth:`from_json`)."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layers: list                 # [HybridLayer]
+    norm_eps: float = 1e-6
+    postln_alpha: float = 1.0
+    max_position: int = 1 << 20  # nothing in the design bounds a sequence; engines pass their own limit
+    arch: str = "pemidra"
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    tie_word_embeddings: bool = False
+
+    MIXERS = ("retention", "general_delta", "parallel")
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_json(cls, d: dict, name: str = "pemidra") -> "PemidraConfig":
+        layers = [HybridLayer(l["type"], dict(l["mixer"]), dict(l["mlp"]) if l.get("mlp") else None)
+                  for l in d["layers"]]
+        for l in layers:
+            if l.type not in cls.MIXERS:
+                raise ValueError(f"unknown mixer type {l.type!r}")
+            if l.mlp is not None and l.mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"unknown feed-forward kind {l.mlp.get('kind')!r}")
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=layers,
+                   norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)), postln_alpha=float(d.get("postln_alpha", 1.0)),
+                   max_position=int(d.get("max_positions", 1 << 20)))
+
+    def to_json(self) -> dict:
+        return {"architecture": "Pemidra", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.norm_eps},
+                "postln_alpha": self.postln_alpha,
+                "layers": [{"type": l.type, "mixer": dict(l.mixer), "mlp": dict(l.mlp) if l.mlp else None}
+                           for l in self.layers]}
+
+
+def pemidra_layers(n: int, heads: int, head_dim: int, ff: int, kv_heads: Optional[int] = None, chunk: int = 256,
+                   rot_dims: Optional[int] = None, lora: int = 64, conv: int = 4,
+                   pattern=("general_delta", "retention", "parallel")) -> list:
+    """``n`` layers cycling through ``pattern`` with one set of head sizes (presets and benchmarks).  Only the
+    ``parallel`` layers carry a feed-forward, as the mixers of the other two are cheap by themselves."""
+    kv = kv_heads or heads
+    out = []
+    for i in range(n):
+        t = pattern[i % len(pattern)]
+        if t == "retention":
+            mixer = {"heads": heads, "dim": head_dim, "vdim": head_dim,
+                     "decay": [1.0 - 2.0 ** (-5 - (j % 8)) for j in range(heads)]}
+        elif t == "general_delta":
+            mixer = {"heads": heads, "dim": head_dim, "lora": lora}
+        else:
+            mixer = {"left": {"heads": heads, "kv_heads": kv, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                              "mask": {"size": chunk}, "rot": {"dims": rot_dims or head_dim, "base": 10000.0}},
+                     "right": {"heads": heads, "kv_heads": kv, "dim": head_dim, "vdim": head_dim, "conv": conv, "lora": lora}}
+        out.append(HybridLayer(t, mixer, {"kind": "dense", "ff": ff} if ff and t == "parallel" else None))
+    return out
+
+
 def lebepel_layers(n: int, hidden: int, heads: int, kv_heads: int, head_dim: int, ff: int, ssm_heads: int, ssm_p: int,
                    ssm_state: int, ssm_groups: int = 1, conv: int = 4, norm_groups: int = 1, pattern=("attention", "mamba2"),
                    scale: Optional[float] = None) -> list:
@@ -184,6 +252,13 @@ DECODERS.update({
                                 max_position=8192, residual_mult=1.0, logit_softcap=30.0),
 })
 
+DECODERS.update({
+    # post-norm linear-state / chunk-attention decoders (random-init presets; checkpoints bring their own config.json)
+    "pemidra-tiny": PemidraConfig("pemidra-tiny", 32768, 128, pemidra_layers(3, 4, 32, 256, kv_heads=2, chunk=24, rot_dims=16,
+                                                                              lora=8), postln_alpha=1.5),
+    "pemidra-1b": PemidraConfig("pemidra-1b", 32768, 2048, pemidra_layers(18, 16, 128, 5632, kv_heads=4), postln_alpha=2.0),
+})
+
 ENCODERS = {
     "bge-base": EncoderConfig("bge-base", "bert", 12, 768, 12, 3072, 30522, pooling="cls"),
     "minilm-l6": EncoderConfig("minilm-l6", "bert", 6, 384, 12, 1536, 30522, pooling="mean"),
@@ -211,6 +286,23 @@ def encoder_config(name: str, **overrides) -> EncoderConfig:
 
 
 def param_count(cfg) -> int:
+    if isinstance(cfg, PemidraConfig):
+        W, n = cfg.hidden, 2 * cfg.vocab_size * cfg.hidden + 2 * cfg.hidden
+        for l in cfg.layers:
+            m = l.mixer
+            if l.type == "retention":
+                n += W * m["heads"] * (2 * m["dim"] + 3 * m["vdim"])
+            elif l.type == "general_delta":
+                hd, r = m["heads"] * m["dim"], m.get("lora", 0)
+                n += 6 * W * hd + r * (W + hd) + 3 * hd
+            else:
+                a, b = m["left"], m["right"]
+                n += W * (a["heads"] * (a["dim"] + 2 * a["vdim"] + 1) + a["kv_heads"] * (a["dim"] + a["vdim"]))
+                r = b.get("lora", 0)
+                n += W * (2 * b["kv_heads"] * b["dim"] + 2 * b["heads"] * b["vdim"] + b["heads"] + 2 * r) \
+                    + r * b["heads"] * (b["dim"] + b["vdim"]) + 2 * W
+            n += 3 * W + (3 * W * l.mlp["ff"] + 3 * W if l.mlp else 0)
+        return n
     if isinstance(cfg, LebepelConfig):
         W, n = cfg.hidden, (cfg.vocab_size * 2 + cfg.max_position + 1) * cfg.hidden
         for l in cfg.layers:

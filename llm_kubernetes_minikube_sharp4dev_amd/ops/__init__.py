@@ -17,7 +17,11 @@ from . import reference as ref
 from ._ext import available, force_reference, lib, use_hip  # noqa: F401
 from .mixers import (conv_silu, embed_pos, gated_group_rmsnorm, linear_swiglu_any, sig_decode_splits,  # noqa: F401
                      sig_prefill_tiles, sigattn_supported, sigmoid_attention_decode, sigmoid_attention_prefill,
-                     softcap, ssm_scan, stream_rmsnorm, unitnorm_kv_write)
+                     softcap, ssm_scan, stream_rmsnorm, unitnorm_kv_write, embed_stream, stream_layernorm, gelu_tanh_mul,
+                     dual_rmsnorm_mean, normrope_kv_write, sink_attention_prefill, sink_attention_decode, mask_first_key,
+                     MASK_CAUSAL, MASK_CHUNK, MASK_WINDOW)
+from .delta import (delta_scan, delta_scan_supported, gated_delta_prep, general_delta_prep, head_norm_gate, tanh_,  # noqa: F401
+                    GATE_SIGMOID, GATE_SILU)
 
 __all__ = [
     "rmsnorm", "layernorm", "embed_layernorm", "silu_mul", "gelu_", "relu_", "rope_kv_",

@@ -22,7 +22,8 @@ from ._ext import lib, use_hip
 
 __all__ = ["embed_pos", "stream_rmsnorm", "softcap", "linear_swiglu_any", "unitnorm_kv_write", "sig_prefill_tiles", "sig_decode_splits",
            "sigmoid_attention_prefill", "sigmoid_attention_decode", "sigattn_supported", "conv_silu", "ssm_scan",
-           "gated_group_rmsnorm"]
+           "gated_group_rmsnorm", "embed_stream", "stream_layernorm", "gelu_tanh_mul", "dual_rmsnorm_mean", "normrope_kv_write",
+           "sink_attention_prefill", "sink_attention_decode", "mask_first_key", "MASK_CAUSAL", "MASK_CHUNK", "MASK_WINDOW"]
 
 SIG_TILE_ROWS = 16       # queries per wave of the prefill kernel
 SIG_MAX_HEAD = 256       # largest per-head q/k or v size the kernels are built for
@@ -273,3 +274,181 @@ def gated_group_rmsnorm(y, z, w, ngroups: int, eps: float):
     v = (y * F.silu(z.float())).view(T, ngroups, inner // ngroups)
     v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
     return (v.reshape(T, inner) * w).to(z.dtype)
+
+
+# ------------------------------------------------------------------ post-norm f32 stream
+def embed_stream(ids, tok, out_dtype=torch.bfloat16):
+    """(x f32 [T, W], h): the token rows as the f32 stream and as the activation-dtype copy the
+    projections read (for f32 activations both are the same tensor)."""
+    if use_hip(tok):
+        x, h = lib().embed_stream(ids, tok, out_dtype)
+        return x, h
+    x = tok[ids.long()].float()
+    return x, (x if out_dtype == torch.float32 else x.to(out_dtype))
+
+
+def stream_layernorm(x, y, ls, alpha: float, w, b, eps: float, out_dtype=torch.bfloat16, idx=None):
+    """Post-norm stream update ``x <- LN(alpha x + ls * y) * w + b`` in place (f32; mean and variance over
+    the row, variance = mean squared deviation) and the activation-dtype copy of the new ``x`` that the
+    next sublayer's projections read (the same tensor for f32 activations).  ``y`` None: a plain layer
+    norm of ``x``.  With ``idx`` (int64 rows) only those rows are normed into a new tensor and ``x``
+    stays as it was (the rows that feed the LM head)."""
+    if use_hip(x):
+        return lib().stream_layernorm(x, y, ls, float(alpha), w, b, float(eps), idx, out_dtype)
+    v = x if idx is None else x.index_select(0, idx)
+    if y is not None:
+        yy = y if idx is None else y.index_select(0, idx)
+        v = alpha * v + (yy.float() * ls if ls is not None else yy.float())
+    mu = v.mean(-1, keepdim=True)
+    d = v - mu
+    r = d / torch.sqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w + b
+    if idx is not None:
+        return r.to(out_dtype)
+    x.copy_(r)
+    return x if out_dtype == torch.float32 else x.to(out_dtype)
+
+
+def gelu_tanh_mul(gu):
+    """[T, 2F] = [gate | up] -> gelu_tanh(gate) * up, [T, F] in the same dtype."""
+    if use_hip(gu):
+        return lib().gelu_tanh_mul(gu)
+    F_ = gu.shape[1] // 2
+    g, u = gu[:, :F_].float(), gu[:, F_:].float()
+    return (F.gelu(g, approximate="tanh") * u).to(gu.dtype)
+
+
+def dual_rmsnorm_mean(a, wa, b, wb, eps: float):
+    """f32 [T, W]: half the sum of ``a`` and ``b``, each first scaled to unit RMS over the row and
+    multiplied by its weight (two branches that read the same input and share one stream update)."""
+    if use_hip(a):
+        return lib().dual_rmsnorm_mean(a, wa, b, wb, float(eps))
+    af, bf = a.float(), b.float()
+    na = af / torch.sqrt(af.pow(2).mean(-1, keepdim=True) + eps) * wa
+    nb = bf / torch.sqrt(bf.pow(2).mean(-1, keepdim=True) + eps) * wb
+    return 0.5 * (na + nb)
+
+
+# ------------------------------------------------------------------ softmax attention with a sink, masked to chunks
+MASK_CAUSAL, MASK_CHUNK, MASK_WINDOW = 0, 1, 2
+
+
+def mask_first_key(qpos: int, mask_kind: int, mask_size: int) -> int:
+    """First position a query at ``qpos`` sees: causal everything, chunk = the start of its chunk of
+    ``mask_size`` positions (counted from position 0 of the sequence), window = the last ``mask_size``."""
+    if mask_kind == MASK_CHUNK:
+        return (qpos // mask_size) * mask_size
+    if mask_kind == MASK_WINDOW:
+        return max(0, qpos - mask_size + 1)
+    return 0
+
+
+def normrope_kv_write(qkv, H: int, G: int, dim: int, vdim: int, q_w, k_w, rot_dims: int, inv_freq, positions, eps: float,
+                      k_cache, v_cache, slots, v_unit: bool = True, norm_dim: Optional[int] = None, norm_vdim: Optional[int] = None):
+    """Rows ``[q: H dim | k: G dim | v: G vdim | ...]``: q and k are RMS-normed per head (f32) with the
+    weights ``q_w`` / ``k_w`` [dim] shared by the heads, then their first ``rot_dims`` dimensions rotated
+    by the row's position (dimension i pairs with i + rot_dims / 2, angle = position * inv_freq[i], f32);
+    v is divided by its RMS per head when ``v_unit``.  q in place, k and v into the paged cache
+    (K ``[blocks, G, BS, dim]``, V key-contiguous ``[blocks, G, vdim, BS]``); slots < 0 cache nothing.
+    ``norm_dim`` / ``norm_vdim``: divisors of the means when heads carry zero padding columns."""
+    norm_dim = dim if norm_dim is None else int(norm_dim)
+    norm_vdim = vdim if norm_vdim is None else int(norm_vdim)
+    if use_hip(qkv):
+        lib().normrope_kv_write(qkv, H, G, dim, vdim, norm_dim, norm_vdim, q_w, k_w, int(rot_dims), inv_freq, positions, float(eps),
+                                k_cache, v_cache, slots, bool(v_unit))
+        return qkv
+    T = qkv.shape[0]
+    half = rot_dims // 2
+    ang = positions[:T].float().view(T, 1, 1) * inv_freq.float().view(1, 1, half)
+    c, s = torch.cos(ang), torch.sin(ang)
+
+    def prep(x, w):
+        x = x / torch.sqrt(x.pow(2).sum(-1, keepdim=True) / norm_dim + eps) * w
+        u, v = x[..., :half].clone(), x[..., half:rot_dims].clone()
+        x[..., :half] = u * c - v * s
+        x[..., half:rot_dims] = v * c + u * s
+        return x
+
+    q = prep(qkv[:, : H * dim].float().view(T, H, dim), q_w)
+    k = prep(qkv[:, H * dim:(H + G) * dim].float().view(T, G, dim), k_w)
+    v = qkv[:, (H + G) * dim:(H + G) * dim + G * vdim].float().view(T, G, vdim)
+    if v_unit:
+        v = v / torch.sqrt(v.pow(2).sum(-1, keepdim=True) / norm_vdim + eps)
+    qkv[:, : H * dim] = q.reshape(T, -1).to(qkv.dtype)
+    BS = k_cache.shape[2]
+    sl = slots[:T].long()
+    ok = sl >= 0
+    blk, off = sl[ok] // BS, sl[ok] % BS
+    k_cache[blk, :, off, :] = k[ok].to(k_cache.dtype)
+    v_cache[blk, :, :, off] = v[ok].to(v_cache.dtype)
+    return qkv
+
+
+def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink):
+    """q f32 [S, H, dim] at positions qpos [S]; k/v f32 [n, G, *] at positions 0..n-1."""
+    H, G = q.shape[1], k.shape[1]
+    rep = H // G
+    s = torch.einsum("ihd,jhd->hij", q, k.repeat_interleave(rep, dim=1)) * hscale.view(-1, 1, 1)
+    j = torch.arange(k.shape[0], device=q.device).view(1, -1)
+    i = qpos.view(-1, 1)
+    if mask_kind == MASK_CHUNK:
+        lo = (i // mask_size) * mask_size
+    elif mask_kind == MASK_WINDOW:
+        lo = (i - mask_size + 1).clamp(min=0)
+    else:
+        lo = torch.zeros_like(i)
+    seen = (j <= i) & (j >= lo)
+    s = s.masked_fill(~seen[None], float("-inf"))
+    m = s.amax(-1, keepdim=True).clamp(min=0.0)          # the sink's score 0 bounds the maximum from below
+    e = torch.exp(s - m)
+    den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sink else 0.0)
+    return torch.einsum("hij,jhd->ihd", e / den, v.repeat_interleave(rep, dim=1))
+
+
+def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H: int, G: int, dim: int, vdim: int, hscale,
+                           mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, tiles=None, q_lens_cpu=None):
+    """Softmax attention of query chunks over their sequences' cached keys inside the mask
+    (``mask_first_key``), with ``sink``: one more term of score 0 and no value in the denominator.
+    ``hscale`` f32 [H]: the score multiplier of each head.  ``gate`` (or None): rows aligned with ``q``
+    whose columns ``gate_col + h`` hold the raw output gate of head h; the head's output is multiplied by
+    its sigmoid.  q: rows whose first H * dim columns are the prepared queries; out [T, H * vdim]."""
+    if use_hip(q):
+        if tiles is None:
+            ql = q_lens_cpu if q_lens_cpu is not None else (cu_q[1:] - cu_q[:-1]).tolist()
+            ts, tq = sig_prefill_tiles(ql, ctx_lens.tolist())
+            tiles = (torch.from_numpy(ts).to(q.device), torch.from_numpy(tq).to(q.device))
+        lib().sinkattn_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, tiles[0], tiles[1], H, G, dim, vdim, hscale,
+                               int(mask_kind), int(mask_size), bool(sink), gate, int(gate_col), out)
+        return out
+    cu = cu_q.tolist()
+    for b in range(len(cu) - 1):
+        s0, s1 = cu[b], cu[b + 1]
+        n = int(ctx_lens[b])
+        k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
+        qq = q[s0:s1, : H * dim].float().view(s1 - s0, H, dim)
+        qpos = torch.arange(n - (s1 - s0), n, device=q.device)
+        o = _sink_rows(qq, k, v, qpos, hscale, mask_kind, mask_size, sink)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[s0:s1, gate_col:gate_col + H].float()).unsqueeze(-1)
+        out[s0:s1, : H * vdim] = o.reshape(s1 - s0, H * vdim).to(out.dtype)
+    return out
+
+
+def sink_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, H: int, G: int, dim: int, vdim: int, hscale,
+                          mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, splits: int = 1, part=None):
+    """One query row per sequence at its last position (ctx - 1) over its cached keys inside the mask."""
+    B = q.shape[0]
+    if use_hip(q):
+        if splits > 1 and part is None:
+            part = torch.empty(B * H * splits * (vdim + 2), dtype=torch.float32, device=q.device)
+        lib().sinkattn_decode(q, k_cache, v_cache, block_tables, ctx_lens, int(splits), H, G, dim, vdim, hscale, int(mask_kind),
+                              int(mask_size), bool(sink), gate, int(gate_col), out, part)
+        return out
+    for b in range(B):
+        n = int(ctx_lens[b])
+        k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
+        qq = q[b:b + 1, : H * dim].float().view(1, H, dim)
+        o = _sink_rows(qq, k, v, torch.tensor([n - 1], device=q.device), hscale, mask_kind, mask_size, sink)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[b:b + 1, gate_col:gate_col + H].float()).unsqueeze(-1)
+        out[b:b + 1, : H * vdim] = o.reshape(1, H * vdim).to(out.dtype)
+    return out
