@@ -24,6 +24,7 @@
 // heads of one kv group (all at the last position).
 #include "common.h"
 #include "kernels.h"
+#include "attn_frag.h"
 
 namespace {
 
@@ -40,36 +41,6 @@ struct SigParams {
   const float* r2;  // [H]
   const float* pb;  // [H]
 };
-
-template <typename T>
-struct El;
-template <>
-struct El<bf16_t> {
-  static constexpr int V = 8;  // elements per 16-byte fragment
-  static LK_DEVICE float ld(const bf16_t* p) { return bf2f(*p); }
-  static LK_DEVICE void st(bf16_t* p, float v) { *p = f2bf(v); }
-};
-template <>
-struct El<float> {
-  static constexpr int V = 4;
-  static LK_DEVICE float ld(const float* p) { return *p; }
-  static LK_DEVICE void st(float* p, float v) { *p = v; }
-};
-
-LK_DEVICE uint4_t ld16(const void* p) { return *reinterpret_cast<const uint4_t*>(p); }
-
-// S^T += A(16 keys x one 16-byte fragment of dims) . B(the columns' same dims)
-template <typename T>
-LK_DEVICE floatx4 mma_qk(uint4_t a, uint4_t b, floatx4 c) {
-  if constexpr (sizeof(T) == 2) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(short8, a), __builtin_bit_cast(short8, b), c, 0, 0, 0);
-  } else {
-    const floatx4 fa = __builtin_bit_cast(floatx4, a), fb = __builtin_bit_cast(floatx4, b);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[e], fb[e], c, 0, 0, 0);
-    return c;
-  }
-}
 
 template <bool EXACT>
 LK_DEVICE float sig_weight(float s, float r1, float r2, float pb, int d) {

@@ -1266,6 +1266,238 @@ at::Tensor gated_group_rmsnorm(const at::Tensor& y, const at::Tensor& z, const a
   return out;
 }
 
+// ---------------------------------------------------------------------------------------------
+// post-norm f32 stream, linear-state scans, softmax attention with a sink (bf16 or f32 activations)
+std::vector<at::Tensor> embed_stream(const at::Tensor& ids, const at::Tensor& tok, at::ScalarType out_dtype) {
+  CHECK_CUDA(ids); CHECK_I32(ids); CHECK_CONTIG(ids); CHECK_CUDA(tok); CHECK_CONTIG(tok);
+  const int esz = esz_of(tok, "tok");
+  TORCH_CHECK(tok.dim() == 2 && tok.scalar_type() == out_dtype, "token table must be [V, W] in the activation dtype");
+  const long T = ids.numel();
+  const int W = tok.size(1);
+  at::Tensor x = at::empty({T, W}, tok.options().dtype(at::kFloat));
+  at::Tensor copy = esz == 2 ? at::empty({T, W}, tok.options()) : x;
+  CHECK_RC(lk_embed_stream(ip(ids), tok.data_ptr(), tok.size(0), T, W, x.data_ptr<float>(), esz == 2 ? copy.data_ptr() : nullptr, esz,
+                           cur_stream()), "embed_stream");
+  return {x, copy};
+}
+
+at::Tensor stream_layernorm(at::Tensor& x, const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& ls, double alpha,
+                            const at::Tensor& w, const at::Tensor& b, double eps, const c10::optional<at::Tensor>& idx,
+                            at::ScalarType out_dtype) {
+  CHECK_CUDA(x); CHECK_F32(x); CHECK_CONTIG(x);
+  TORCH_CHECK(x.dim() == 2, "x must be [T, W]");
+  TORCH_CHECK(out_dtype == at::kBFloat16 || out_dtype == at::kFloat, "out dtype");
+  const long T = x.size(0);
+  const int W = x.size(1);
+  long ys = 0;
+  int yesz = 4;
+  if (y) {
+    CHECK_CUDA(*y); CHECK_LASTDIM(*y);
+    yesz = esz_of(*y, "y");
+    TORCH_CHECK(y->dim() == 2 && y->size(0) == T && y->size(1) == W, "y shape");
+    ys = y->stride(0);
+  }
+  if (idx) { CHECK_CUDA(*idx); TORCH_CHECK(idx->scalar_type() == at::kLong && idx->is_contiguous(), "idx must be int64"); }
+  // in place: f32 activations read x itself; rows chosen by idx always go to a new tensor
+  const bool copy = idx || out_dtype == at::kBFloat16;
+  at::Tensor out = copy ? at::empty({idx ? idx->numel() : T, W}, x.options().dtype(out_dtype)) : x;
+  CHECK_RC(lk_stream_layernorm(x.data_ptr<float>(), y ? y->data_ptr() : nullptr, ys, yesz, fpo(ls, W, "ls"), (float)alpha,
+                               fp(w, W, "w"), fp(b, W, "b"), (float)eps, idx ? idx->data_ptr<int64_t>() : nullptr, out.size(0),
+                               copy ? out.data_ptr() : nullptr, out.stride(0), (int)out.element_size(), W, cur_stream()),
+           "stream_layernorm");
+  return out;
+}
+
+at::Tensor gelu_tanh_mul(const at::Tensor& gu) {
+  CHECK_CUDA(gu); CHECK_LASTDIM(gu);
+  const int esz = esz_of(gu, "gu");
+  TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0, "gu must be [T, 2 F]");
+  const int F = gu.size(1) / 2;
+  at::Tensor out = at::empty({gu.size(0), F}, gu.options());
+  CHECK_RC(lk_gelu_tanh_mul(gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), gu.size(0), F, esz, cur_stream()),
+           "gelu_tanh_mul");
+  return out;
+}
+
+at::Tensor dual_rmsnorm_mean(const at::Tensor& a, const at::Tensor& wa, const at::Tensor& b, const at::Tensor& wb, double eps) {
+  CHECK_CUDA(a); CHECK_CUDA(b); CHECK_LASTDIM(a); CHECK_LASTDIM(b);
+  const int esz = esz_of(a, "a");
+  same_type(b, a, "b");
+  TORCH_CHECK(a.dim() == 2 && b.dim() == 2 && a.sizes() == b.sizes(), "a / b shape");
+  const int W = a.size(1);
+  at::Tensor out = at::empty({a.size(0), W}, a.options().dtype(at::kFloat));
+  CHECK_RC(lk_dual_rmsnorm_mean(a.data_ptr(), a.stride(0), fp(wa, W, "wa"), b.data_ptr(), b.stride(0), fp(wb, W, "wb"), (float)eps,
+                                out.data_ptr<float>(), a.size(0), W, esz, cur_stream()), "dual_rmsnorm_mean");
+  return out;
+}
+
+// rows of a 2-d tensor with at least n columns, contiguous along the row
+void check_rows(const at::Tensor& t, long T, long n, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.size(0) == T && t.size(1) >= n && t.stride(1) == 1, name, " must be GPU rows of >= ", n);
+}
+const float* f32_rows(const c10::optional<at::Tensor>& t, long T, long n, const char* name, long* stride) {
+  if (!t) return nullptr;
+  check_rows(*t, T, n, name);
+  TORCH_CHECK(t->scalar_type() == at::kFloat, name, " must be float32");
+  *stride = t->stride(0);
+  return t->data_ptr<float>();
+}
+
+at::Tensor delta_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& w,
+                      const c10::optional<at::Tensor>& p, const c10::optional<at::Tensor>& z, at::Tensor& state, const at::Tensor& cu,
+                      const at::Tensor& slots, const at::Tensor& positions, int64_t H, int64_t Hk, int64_t dk, int64_t dv,
+                      const c10::optional<at::Tensor>& w_head, double k_scale, int64_t max_len) {
+  const long T = q.size(0);
+  TORCH_CHECK(H >= 1 && Hk >= 1 && H % Hk == 0 && dk >= 1 && dk <= 256 && dv >= 1, "delta_scan sizes");
+  check_rows(q, T, Hk * dk, "q"); check_rows(k, T, Hk * dk, "k"); check_rows(v, T, H * dv, "v");
+  const int esz = esz_of(q, "q");
+  same_type(k, q, "k"); same_type(v, q, "v");
+  long ws = 0, ps = 0, zs = 0;
+  const float* wp = f32_rows(w, T, H * dk, "w", &ws);
+  const float* pp = f32_rows(p, T, H * dk, "p", &ps);
+  const float* zp = f32_rows(z, T, H * dk, "z", &zs);
+  TORCH_CHECK((wp != nullptr) == (pp != nullptr) && (pp != nullptr) == (zp != nullptr), "w, p, z come together (or none, with w_head)");
+  TORCH_CHECK(wp != nullptr || w_head.has_value(), "w or w_head");
+  check_seqs(cu, slots, positions, T);
+  CHECK_CUDA(state); CHECK_F32(state); CHECK_CONTIG(state);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk && state.size(3) == dv, "state must be f32 [slots, H, dk, dv]");
+  at::Tensor o = at::empty({T, H * dv}, q.options().dtype(at::kFloat));
+  CHECK_RC(lk_delta_scan(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), esz, wp, ws, pp, ps, zp, zs,
+                         wp ? nullptr : fpo(w_head, H, "w_head"), (float)k_scale, state.data_ptr<float>(), ip(cu), ip(slots),
+                         ip(positions), cu.numel() - 1, (int)H, (int)Hk, (int)dk, (int)dv, o.data_ptr<float>(), o.stride(0),
+                         cur_stream()), "delta_scan");
+  return o;
+}
+
+std::vector<at::Tensor> gated_delta_prep(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& beta,
+                                         const at::Tensor& dt, const at::Tensor& dt_bias, const at::Tensor& A_log, int64_t H,
+                                         int64_t Hk, int64_t dk, int64_t dv) {
+  const long T = q.size(0);
+  TORCH_CHECK(H >= 1 && Hk >= 1 && H % Hk == 0, "heads");
+  check_rows(q, T, Hk * dk, "q"); check_rows(k, T, Hk * dk, "k"); check_rows(v, T, H * dv, "v");
+  check_rows(beta, T, H, "beta"); check_rows(dt, T, H * dk, "dt");
+  const int esz = esz_of(q, "q");
+  same_type(k, q, "k"); same_type(v, q, "v"); same_type(beta, q, "beta"); same_type(dt, q, "dt");
+  auto f = q.options().dtype(at::kFloat);
+  at::Tensor qn = at::empty({T, Hk * dk}, f), kn = at::empty({T, Hk * dk}, f), vb = at::empty({T, H * dv}, f);
+  at::Tensor g = at::empty({T, H * dk}, f), p = at::empty({T, H * dk}, f), z = at::empty({T, H * dk}, f);
+  CHECK_RC(lk_gated_delta_prep(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), beta.data_ptr(),
+                               beta.stride(0), dt.data_ptr(), dt.stride(0), fp(dt_bias, H * dk, "dt_bias"), fp(A_log, H, "A_log"), T,
+                               (int)H, (int)Hk, (int)dk, (int)dv, qn.data_ptr<float>(), kn.data_ptr<float>(), vb.data_ptr<float>(),
+                               g.data_ptr<float>(), p.data_ptr<float>(), z.data_ptr<float>(), esz, cur_stream()), "gated_delta_prep");
+  return {qn, kn, vb, g, p, z};
+}
+
+std::vector<at::Tensor> general_delta_prep(const at::Tensor& k, const at::Tensor& wraw, const at::Tensor& w0, const at::Tensor& araw,
+                                           const at::Tensor& a_b, int64_t H, int64_t dk) {
+  const long T = k.size(0);
+  check_rows(k, T, H * dk, "k"); check_rows(wraw, T, H * dk, "wraw"); check_rows(araw, T, H * dk, "araw");
+  const int esz = esz_of(k, "k");
+  same_type(wraw, k, "wraw"); same_type(araw, k, "araw");
+  auto f = k.options().dtype(at::kFloat);
+  at::Tensor w = at::empty({T, H * dk}, f), p = at::empty({T, H * dk}, f), z = at::empty({T, H * dk}, f);
+  CHECK_RC(lk_general_delta_prep(k.data_ptr(), k.stride(0), wraw.data_ptr(), wraw.stride(0), fp(w0, H * dk, "w0"), araw.data_ptr(),
+                                 araw.stride(0), fp(a_b, H * dk, "a_b"), T, (int)H, (int)dk, w.data_ptr<float>(), p.data_ptr<float>(),
+                                 z.data_ptr<float>(), esz, cur_stream()), "general_delta_prep");
+  return {w, p, z};
+}
+
+at::Tensor head_norm_gate(const at::Tensor& o, const at::Tensor& gate, const c10::optional<at::Tensor>& w, int64_t H, double eps,
+                          int64_t kind, at::ScalarType out_dtype) {
+  CHECK_CUDA(o); CHECK_F32(o); CHECK_LASTDIM(o);
+  TORCH_CHECK(o.dim() == 2 && H >= 1 && o.size(1) % H == 0, "o must be [T, H dv]");
+  TORCH_CHECK(out_dtype == at::kBFloat16 || out_dtype == at::kFloat, "out dtype");
+  const long T = o.size(0), n = o.size(1);
+  check_rows(gate, T, n, "gate");
+  const int gesz = esz_of(gate, "gate");
+  at::Tensor out = at::empty({T, n}, o.options().dtype(out_dtype));
+  CHECK_RC(lk_head_norm_gate(o.data_ptr<float>(), o.stride(0), gate.data_ptr(), gate.stride(0), gesz, fpo(w, n, "w"), T, (int)H,
+                             (int)(n / H), (float)eps, (int)kind, out.data_ptr(), out.stride(0), (int)out.element_size(), cur_stream()),
+           "head_norm_gate");
+  return out;
+}
+
+void tanh_(at::Tensor& x) {
+  CHECK_CUDA(x); CHECK_LASTDIM(x);
+  TORCH_CHECK(x.dim() == 2, "x must be 2-d");
+  CHECK_RC(lk_tanh_(x.data_ptr(), x.stride(0), x.size(0), (int)x.size(1), esz_of(x, "x"), cur_stream()), "tanh_");
+}
+
+void normrope_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64_t vdim, int64_t norm_dim, int64_t norm_vdim,
+                       const at::Tensor& qw, const at::Tensor& kw, int64_t rot, const at::Tensor& inv_freq, const at::Tensor& positions,
+                       double eps, at::Tensor& kc, at::Tensor& vc, const at::Tensor& slots, bool v_unit) {
+  CHECK_CUDA(qkv); CHECK_LASTDIM(qkv); CHECK_I32(slots); CHECK_CONTIG(slots); CHECK_CUDA(positions); CHECK_I32(positions);
+  CHECK_CONTIG(positions);
+  const int esz = esz_of(qkv, "qkv");
+  const long T = qkv.size(0);
+  TORCH_CHECK(qkv.dim() == 2 && qkv.size(1) >= (H + G) * dim + G * vdim, "qkv must be [T, >= (H + G) dim + G vdim]");
+  TORCH_CHECK(slots.numel() >= T && positions.numel() >= T, "slots / positions");
+  TORCH_CHECK(rot >= 0 && rot % 2 == 0 && rot <= dim, "rot");
+  check_sig_caches(qkv, kc, vc, G, dim, vdim);
+  CHECK_RC(lk_normrope_kv_write(qkv.data_ptr(), qkv.stride(0), T, (int)H, (int)G, (int)dim, (int)vdim, (int)norm_dim, (int)norm_vdim,
+                                fp(qw, dim, "q norm weight"), fp(kw, dim, "k norm weight"), (int)rot,
+                                fp(inv_freq, std::max<int64_t>(rot / 2, 1), "inv_freq"), ip(positions), (float)eps, kc.data_ptr(),
+                                vc.data_ptr(), ip(slots), (int)kc.size(2), v_unit ? 1 : 0, esz, cur_stream()), "normrope_kv_write");
+}
+
+const void* gate_rows(const c10::optional<at::Tensor>& gate, const at::Tensor& q, int64_t gate_col, int64_t H, long* gs) {
+  if (!gate) return nullptr;
+  check_rows(*gate, q.size(0), gate_col + H, "gate");
+  same_type(*gate, q, "gate");
+  TORCH_CHECK(gate_col >= 0, "gate_col");
+  *gs = gate->stride(0);
+  return gate->data_ptr();
+}
+
+void sinkattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt, const at::Tensor& cu_q,
+                      const at::Tensor& ctx, const at::Tensor& tile_seq, const at::Tensor& tile_q0, int64_t H, int64_t G, int64_t dim,
+                      int64_t vdim, const at::Tensor& hscale, int64_t mkind, int64_t msize, bool sink,
+                      const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out) {
+  CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(out); CHECK_LASTDIM(out);
+  const int esz = esz_of(q, "q");
+  same_type(out, q, "out");
+  TORCH_CHECK(q.dim() == 2 && q.size(1) >= H * dim && out.dim() == 2 && out.size(0) == q.size(0) && out.size(1) >= H * vdim, "q / out shape");
+  check_rows16(q, "q");
+  check_sig_caches(q, kc, vc, G, dim, vdim);
+  CHECK_CUDA(bt); CHECK_I32(bt); CHECK_I32(cu_q); CHECK_I32(ctx); CHECK_I32(tile_seq); CHECK_I32(tile_q0);
+  CHECK_CONTIG(cu_q); CHECK_CONTIG(ctx); CHECK_CONTIG(tile_seq); CHECK_CONTIG(tile_q0);
+  TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1 && bt.size(0) >= cu_q.numel() - 1 && ctx.numel() >= cu_q.numel() - 1 &&
+              tile_q0.numel() == tile_seq.numel(), "block tables / lengths / tiles");
+  long gs = 0;
+  const void* gp = gate_rows(gate, q, gate_col, H, &gs);
+  CHECK_RC(lk_sinkattn_prefill(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), (int)bt.stride(0), ip(cu_q), ip(ctx),
+                               ip(tile_seq), ip(tile_q0), (int)tile_seq.numel(), (int)H, (int)G, (int)dim, (int)vdim, (int)kc.size(2),
+                               fp(hscale, H, "hscale"), (int)mkind, (int)msize, sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(),
+                               out.stride(0), esz, cur_stream()), "sinkattn_prefill");
+}
+
+void sinkattn_decode(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt, const at::Tensor& ctx,
+                     int64_t Z, int64_t H, int64_t G, int64_t dim, int64_t vdim, const at::Tensor& hscale, int64_t mkind,
+                     int64_t msize, bool sink, const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out,
+                     const c10::optional<at::Tensor>& part) {
+  CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(out); CHECK_LASTDIM(out);
+  const int esz = esz_of(q, "q");
+  same_type(out, q, "out");
+  const long B = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) >= H * dim && out.dim() == 2 && out.size(0) == B && out.size(1) >= H * vdim, "q / out shape");
+  check_rows16(q, "q");
+  check_sig_caches(q, kc, vc, G, dim, vdim);
+  CHECK_CUDA(bt); CHECK_I32(bt); CHECK_I32(ctx); CHECK_CONTIG(ctx);
+  TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1 && bt.size(0) >= B && ctx.numel() >= B && Z >= 1 && Z <= 65535, "block tables / lengths / splits");
+  float* pp = nullptr;
+  if (Z > 1) {
+    TORCH_CHECK(part.has_value() && part->is_cuda() && part->scalar_type() == at::kFloat && part->is_contiguous() &&
+                part->numel() >= B * H * Z * (vdim + 2), "part must be f32 [B, H, Z, vdim + 2]");
+    pp = part->data_ptr<float>();
+  }
+  long gs = 0;
+  const void* gp = gate_rows(gate, q, gate_col, H, &gs);
+  CHECK_RC(lk_sinkattn_decode(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), (int)bt.stride(0), ip(ctx), (int)B, (int)Z,
+                              (int)H, (int)G, (int)dim, (int)vdim, (int)kc.size(2), fp(hscale, H, "hscale"), (int)mkind, (int)msize,
+                              sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(), out.stride(0), pp, esz, cur_stream()),
+           "sinkattn_decode");
+}
+
 }  // namespace
 // build provenance: "LKSTAMP:<hash of sources + flags>", generated by csrc/build.py at link time
 extern "C" const char lk_source_stamp[];
@@ -1285,6 +1517,18 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("conv_silu", &conv_silu);
   m.def("ssm_scan", &ssm_scan);
   m.def("gated_group_rmsnorm", &gated_group_rmsnorm);
+  m.def("embed_stream", &embed_stream);
+  m.def("stream_layernorm", &stream_layernorm);
+  m.def("gelu_tanh_mul", &gelu_tanh_mul);
+  m.def("dual_rmsnorm_mean", &dual_rmsnorm_mean);
+  m.def("delta_scan", &delta_scan);
+  m.def("gated_delta_prep", &gated_delta_prep);
+  m.def("general_delta_prep", &general_delta_prep);
+  m.def("head_norm_gate", &head_norm_gate);
+  m.def("tanh_", &tanh_);
+  m.def("normrope_kv_write", &normrope_kv_write);
+  m.def("sinkattn_prefill", &sinkattn_prefill);
+  m.def("sinkattn_decode", &sinkattn_decode);
   m.def("window_mark", [](int64_t id) { CHECK_RC(lk_window_mark((int)id, cur_stream()), "window_mark"); });
   m.def("debug_invalid_launch", []() { CHECK_RC(lk_debug_invalid_launch(cur_stream()), "debug_invalid_launch"); });
   // a HIP stream restricted to the CUs of a bit mask (32 CUs per word): two kernels that

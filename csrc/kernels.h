@@ -250,3 +250,40 @@ int lk_ssm_scan(const void* xbc, long xs, const void* dt, long dts, int S, int h
                 const int* positions, float* y, long ys, int max_len, int esz, hipStream_t st);
 int lk_gated_group_rmsnorm(const float* y, long ys, const void* z, long zs, const float* w, long rows, int inner,
                            int ngroups, float eps, void* out, long os, int esz, hipStream_t st);
+
+// csrc/stream_ln.hip: post-norm f32 stream (x <- LN(alpha x + ls * y) * w + b with an activation-dtype copy), token gather,
+// gated tanh-GELU of a fused [gate | up] projection, mean of two RMS-normed branches
+int lk_embed_stream(const int* ids, const void* tok, long V, long T, int W, float* x, void* copy, int esz, hipStream_t st);
+int lk_stream_layernorm(float* x, const void* y, long ys, int y_esz, const float* ls, float alpha, const float* w, const float* b,
+                        float eps, const long* idx, long rows, void* out, long os, int out_esz, int W, hipStream_t st);
+int lk_gelu_tanh_mul(const void* gu, long gs, void* out, long os, long rows, int F, int esz, hipStream_t st);
+int lk_dual_rmsnorm_mean(const void* a, long as, const float* wa, const void* b, long bs, const float* wb, float eps, float* out,
+                         long rows, int W, int esz, hipStream_t st);
+
+// csrc/delta_scan.hip: S_t = diag(w_t) S_(t-1) - p_t (z_t^T S_(t-1)) + k_t v_t^T, o_t = S_t^T q_t over per-sequence state slots
+// (state f32 [slots, H, dk, dv]); operand preparation of the gated and the generalized delta rule; per-head RMS norm with a gate
+int lk_delta_scan(const void* q, long qs, const void* k, long ks, const void* v, long vs, int qkv_esz, const float* w, long ws,
+                  const float* p, long ps, const float* z, long zs, const float* w_head, float k_scale, float* state,
+                  const int* cu, const int* slots, const int* positions, int S, int H, int Hk, int dk, int dv, float* o, long os,
+                  hipStream_t st);
+int lk_gated_delta_prep(const void* q, long qs, const void* k, long ks, const void* v, long vs, const void* beta, long bs,
+                        const void* dt, long dts, const float* dt_bias, const float* A_log, long T, int H, int Hk, int dk, int dv,
+                        float* qn, float* kn, float* vb, float* g, float* p, float* z, int esz, hipStream_t st);
+int lk_general_delta_prep(const void* k, long ks, const void* wraw, long wrs, const float* w0, const void* araw, long ars,
+                          const float* a_b, long T, int H, int dk, float* w, float* p, float* z, int esz, hipStream_t st);
+int lk_head_norm_gate(const float* o, long os, const void* g, long gs, int g_esz, const float* w, long T, int H, int dv, float eps,
+                      int kind, void* out, long outs, int out_esz, hipStream_t st);
+int lk_tanh_(void* x, long xs, long T, int n, int esz, hipStream_t st);
+
+// csrc/attn_sink.hip: softmax attention with a sink and a position mask (0 causal, 1 chunks, 2 window) over the paged caches
+// K [NB, G, BS, dim], V [NB, G, vdim, BS]; q / k RMS norm + partial rotation, v norm and the cache write
+int lk_normrope_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, int norm_dim, int norm_vdim, const float* qw,
+                         const float* kw, int rot, const float* inv_freq, const int* positions, float eps, void* kc, void* vc,
+                         const int* slots, int BS, int v_unit, int esz, hipStream_t st);
+int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* cu_q,
+                        const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H, int G, int dim, int vdim,
+                        int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol, void* out,
+                        long os, int esz, hipStream_t st);
+int lk_sinkattn_decode(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* ctx_lens,
+                       int B, int Z, int H, int G, int dim, int vdim, int BS, const float* hscale, int mkind, int msize, int sink,
+                       const void* gate, long gs, int gcol, void* out, long os, float* part, int esz, hipStream_t st);
