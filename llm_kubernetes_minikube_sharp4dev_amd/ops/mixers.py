@@ -358,7 +358,7 @@ def normrope_kv_write(qkv, H: int, G: int, dim: int, vdim: int, q_w, k_w, rot_di
         return qkv
     T = qkv.shape[0]
     half = rot_dims // 2
-    ang = positions[:T].float().view(T, 1, 1) * inv_freq.float().view(1, 1, half)
+    ang = positions[:T].float().view(T, 1, 1) * inv_freq.float()[:half].view(1, 1, half)
     c, s = torch.cos(ang), torch.sin(ang)
 
     def prep(x, w):
