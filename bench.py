@@ -141,9 +141,9 @@ def parse():
                          "(benchmarks/xgmi_floor.py --world 2; default profiles/r4_tp_collectives/floor_tp2_h<H>.json)")
     ap.add_argument("--json-out", default=None)
     ap.add_argument("--decoder-bench", action="store_true",
-                    help="instead of the headline workload: prefill and decode tokens/s of the hybrid Lebepel decoder "
-                         "beside a Llama decoder of equal size at a few layer sizes (benchmarks/decoder_bench.py; "
-                         "its own options follow after --)")
+                    help="instead of the headline workload: prefill and decode tokens/s of the hybrid decoders "
+                         "(Lebepel by default; Pemidra with -- --models pemidra,lebepel,llama) beside a Llama decoder of "
+                         "equal size at a few layer sizes (benchmarks/decoder_bench.py; its own options follow after --)")
     args, rest = ap.parse_known_args()
     if rest and not args.decoder_bench:
         ap.error(f"unrecognized arguments: {' '.join(rest)}")

@@ -1,10 +1,10 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of the hybrid Lebepel decoder beside a Llama decoder of the same
-width, depth, heads, head size, feed-forward and vocabulary (random weights, bf16, one GPU), both
-through the same engine: prefill = S fresh prompts of L tokens in one step, decode = B sequences at
+"""Prefill and decode throughput of the hybrid decoders (Lebepel; Pemidra with ``--models pemidra,lebepel``)
+beside a Llama decoder of the same width, depth, heads, head size, feed-forward and vocabulary (random
+weights, bf16, one GPU), all through the same engine: prefill = S fresh prompts of L tokens in one step, decode = B sequences at
 context C, one token each per step (hipGraph replay).  ``bench.py --decoder-bench`` runs this.
 
-    python benchmarks/decoder_bench.py [--sizes 1024,2048,4096] [--json-out FILE]
+    python benchmarks/decoder_bench.py [--sizes 1024,2048,4096] [--models lebepel,llama] [--json-out FILE]
 
 One JSON line per (size, model), then a table.  Per-kernel times come from running it under
 ``rocprofv3 --kernel-trace --stats`` with ``--sizes`` set to one size.
@@ -32,12 +32,18 @@ VOCAB = 32768
 
 def models(width: int, which: str, device):
     from llm_kubernetes_minikube_sharp4dev_amd.models import build_decoder
-    from llm_kubernetes_minikube_sharp4dev_amd.models.configs import LebepelConfig, decoder_config, lebepel_layers
+    from llm_kubernetes_minikube_sharp4dev_amd.models.configs import (LebepelConfig, PemidraConfig, decoder_config, lebepel_layers,
+                                                                      pemidra_layers)
 
     L, H, G, D, FF, sh, sp, sn, sg = SIZES[width]
     if which == "lebepel":
         cfg = LebepelConfig(f"lebepel-w{width}", VOCAB, width, lebepel_layers(L, width, H, G, D, FF, sh, sp, sn, sg, 4, sg),
                             max_position=8192, residual_mult=0.5, logit_softcap=30.0)
+    elif which == "pemidra":
+        # general_delta / retention / parallel (attention in chunks of 256 beside a gated delta rule, with the
+        # feed-forward) in turn; the same heads and head size for every mixer, two-layer projections of rank 128
+        cfg = PemidraConfig(f"pemidra-w{width}", VOCAB, width, pemidra_layers(L, H, D, FF, kv_heads=G, chunk=256, lora=128),
+                            postln_alpha=2.0)
     else:
         cfg = decoder_config("llama-3-8b", num_layers=L, hidden=width, num_heads=H, num_kv_heads=G, head_dim=D,
                              intermediate=FF, vocab_size=VOCAB, max_position=8192)
@@ -94,7 +100,7 @@ def run(width: int, which: str, a) -> dict:
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--sizes", default="1024,2048,4096")
-    ap.add_argument("--models", default="lebepel,llama")
+    ap.add_argument("--models", default="lebepel,llama", help="comma list of lebepel, pemidra, llama")
     ap.add_argument("--prefill-seqs", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=1024)
     ap.add_argument("--decode-batch", type=int, default=64)

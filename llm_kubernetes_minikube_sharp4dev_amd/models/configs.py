@@ -182,7 +182,7 @@ class PemidraConfig:
 
 
 def pemidra_layers(n: int, heads: int, head_dim: int, ff: int, kv_heads: Optional[int] = None, chunk: int = 256,
-                   rot_dims: Optional[int] = None, lora: int = 64, conv: int = 4,
+                   rot_dims: Optional[int] = None, lora: int = 128, conv: int = 4,
                    pattern=("general_delta", "retention", "parallel")) -> list:
     """``n`` layers cycling through ``pattern`` with one set of head sizes (presets and benchmarks).  Only the
     ``parallel`` layers carry a feed-forward, as the mixers of the other two are cheap by themselves."""
