@@ -201,19 +201,26 @@ LK_DEVICE float gate_of(const SinkParams& p, long row, int head) {
   return 1.f / (1.f + expf(-gv));
 }
 
-// ---- prefill: workgroup = one 16-query tile of one head; blockIdx.x = head, blockIdx.y walks the tile list
-template <typename T, int PAD>
+// ---- prefill: blockIdx.x = head, blockIdx.y walks the tile list (16 queries of one sequence each).
+// WT = false: a workgroup owns one tile, its 4 waves take every fourth 32-key step and are merged (long key
+// ranges: the chain of steps is what bounds the tile).  WT = true: each wave owns a tile of its own and
+// walks all its steps (masks that bound a query's keys to a few steps: no merge and no barrier; the four
+// tiles of a workgroup are neighbours in the cost-sorted tile list, so its waves finish together).
+template <typename T, int PAD, bool WT>
 __global__ __launch_bounds__(256) void sinkattn_prefill_kernel(SinkParams p, const int* __restrict__ cu_q,
                                                                const int* __restrict__ ctx_lens,
                                                                const int* __restrict__ tile_seq,
-                                                               const int* __restrict__ tile_q0, T* __restrict__ out, long os) {
-  constexpr int VT = PAD / 16;
+                                                               const int* __restrict__ tile_q0, int ntiles, T* __restrict__ out,
+                                                               long os) {
+  constexpr int VT = PAD / 16, NR = WT ? 1 : 3;
   constexpr bool EXACT = sizeof(T) == 4;
-  __shared__ float red[3][VT][64][4];
-  __shared__ float ml[3][64][2];
+  __shared__ float red[NR][VT][64][4];
+  __shared__ float ml[NR][64][2];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, n16 = lane & 15, g = lane >> 4;
   const int head = blockIdx.x;
-  const int b = tile_seq[blockIdx.y], q0 = tile_q0[blockIdx.y];
+  const int tile = WT ? blockIdx.y * 4 + w : blockIdx.y;
+  if (WT && tile >= ntiles) return;   // wave-uniform; no barrier follows in this mode
+  const int b = tile_seq[tile], q0 = tile_q0[tile];
   const int qbeg = cu_q[b], qlen = cu_q[b + 1] - qbeg, ctx = ctx_lens[b], past = ctx - qlen;
   const int qi = q0 + n16;
   const bool cvalid = qi < qlen;
@@ -227,10 +234,15 @@ __global__ __launch_bounds__(256) void sinkattn_prefill_kernel(SinkParams p, con
   float m = p.sink ? 0.f : kNegBig, l = 0.f;
   const int k1 = min(ctx, past + q0 + 16);
   const int k0 = first_key(past + q0, p.mkind, p.msize) & ~31;   // first(i) never decreases with i
-  sink_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, k0, k1, w, 4, cvalid, qpos,
+  sink_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, k0, k1, WT ? 0 : w, WT ? 1 : 4, cvalid, qpos,
                    first_key(qpos, p.mkind, p.msize), p.hscale[head], m, l, o);
-  merge_waves<EXACT, VT>(m, l, o, red, ml);
-  if (w == 0 && cvalid) {
+  if constexpr (WT) {
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+  } else {
+    merge_waves<EXACT, VT>(m, l, o, red, ml);
+  }
+  if ((WT || w == 0) && cvalid) {
     const float den = l + (p.sink ? exp_f<EXACT>(-m) : 0.f);
     const float f = den > 0.f ? gate_of<T>(p, qbeg + qi, head) / den : 0.f;
     T* orow = out + (long)(qbeg + qi) * os + (long)head * p.vdim;
@@ -414,8 +426,12 @@ bool shape_ok(const SinkParams& p, int esz) {
 template <typename T, int PAD>
 int launch_prefill(const SinkParams& p, const int* cu_q, const int* ctx, const int* ts, const int* tq, int ntiles, void* out,
                    long os, hipStream_t st) {
-  if (ntiles > 65535) return -2;
-  sinkattn_prefill_kernel<T, PAD><<<dim3(p.H, ntiles), 256, 0, st>>>(p, cu_q, ctx, ts, tq, reinterpret_cast<T*>(out), os);
+  // a query that sees at most 512 keys (17 steps): one wave per tile
+  const bool wt = p.mkind != 0 && p.msize <= 512;
+  const int gy = wt ? (ntiles + 3) / 4 : ntiles;
+  if (gy > 65535) return -2;
+  if (wt) sinkattn_prefill_kernel<T, PAD, true><<<dim3(p.H, gy), 256, 0, st>>>(p, cu_q, ctx, ts, tq, ntiles, reinterpret_cast<T*>(out), os);
+  else sinkattn_prefill_kernel<T, PAD, false><<<dim3(p.H, gy), 256, 0, st>>>(p, cu_q, ctx, ts, tq, ntiles, reinterpret_cast<T*>(out), os);
   LK_CHECK_LAUNCH();
   return 0;
 }

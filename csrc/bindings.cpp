@@ -1362,10 +1362,13 @@ at::Tensor delta_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
   CHECK_CUDA(state); CHECK_F32(state); CHECK_CONTIG(state);
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk && state.size(3) == dv, "state must be f32 [slots, H, dk, dv]");
   at::Tensor o = at::empty({T, H * dv}, q.options().dtype(at::kFloat));
+  // few (sequence, head) pairs: 16 lanes per state column instead of 4 (a static function of the step's shape)
+  const long S = cu.numel() - 1;
+  const int wide = S * H * ((dv * 4 + 255) / 256) < 2 * 256 ? 1 : 0;
   CHECK_RC(lk_delta_scan(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), esz, wp, ws, pp, ps, zp, zs,
                          wp ? nullptr : fpo(w_head, H, "w_head"), (float)k_scale, state.data_ptr<float>(), ip(cu), ip(slots),
                          ip(positions), cu.numel() - 1, (int)H, (int)Hk, (int)dk, (int)dv, o.data_ptr<float>(), o.stride(0),
-                         cur_stream()), "delta_scan");
+                         wide, cur_stream()), "delta_scan");
   return o;
 }
 

@@ -13,9 +13,11 @@
 //
 // Scan kernel: a workgroup owns (sequence, head, a block of state columns).  A state column is split
 // over R adjacent lanes, each holding DKT of its rows in registers for the whole sequence; the two
-// contractions over the rows (z^T S and q^T S) are finished with R - 1 lane shuffles, so nothing but the
-// tile staging needs a barrier.  The operands of a tile of tokens are staged in LDS as f32 (each row
+// contractions over the rows (z^T S and q^T S) are finished with log2(R) cross-lane moves, so nothing but
+// the tile staging needs a barrier.  The operands of a tile of tokens are staged in LDS as f32 (each row
 // slice padded by 4 floats, so the R different 16-byte broadcasts of one read hit different banks).
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -54,18 +56,42 @@ struct ScanParams {
   int H, Hk, dk, dv;
 };
 
-template <int DKT>
-constexpr int tile_tokens() { return DKT >= 64 ? 8 : 16; }
+// tokens per LDS tile: as many (16 at most, 4 at least) as keep the operands of a tile near 48 KB
+template <int NOPS, int ROW>
+constexpr int tile_tokens() {
+  return NOPS * ROW * 4 * 16 <= 49152 ? 16 : NOPS * ROW * 4 * 8 <= 53248 ? 8 : 4;
+}
+
+// Sum over the R adjacent lanes that share a state column (R a power of two up to 16, groups aligned
+// to R): data-parallel-primitive moves inside a row of 16 lanes, no LDS round trip.
+template <int R>
+LK_DEVICE float group_sum(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  if constexpr (R >= 2) v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1, 0, 3, 2]
+  if constexpr (R >= 4) v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2, 3, 0, 1]
+  if constexpr (R >= 8) v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror: the other quad of 8
+  if constexpr (R >= 16) v += dpp(v, std::integral_constant<int, 0x140>{});  // row_mirror: the other half of 16
+  return v;
+}
+
+template <int DKT, int NOPS>
+struct TokenOps {
+  floatx4 v[NOPS][DKT / 4];
+  float vj;
+};
 
 // FULL: w per channel and the removal term; !FULL: w_head, no removal.
 template <typename TQ, int DKT, int R, bool FULL>
 __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
-  constexpr int TT = tile_tokens<DKT>(), ROW = R * (DKT + 4), NOPS = FULL ? 5 : 2;
+  constexpr int ROW = R * (DKT + 4), NOPS = FULL ? 5 : 2, TT = tile_tokens<NOPS, ROW>();
   constexpr int OQ = 0, OK = 1, OW = 2, OP = 3, OZ = 4;
+  constexpr bool PREFETCH = DKT <= 16;   // the next token's operands are read while this one is computed
   __shared__ __attribute__((aligned(16))) float ops[TT][NOPS][ROW];
   __shared__ float vs[TT][256 / R];
   const int s = blockIdx.x, h = blockIdx.y;
-  const int cols = blockDim.x / R;  // state columns of this workgroup
+  constexpr int cols = 256 / R;  // state columns of this workgroup (256 threads)
   const int j0 = blockIdx.z * cols;
   const int r = threadIdx.x % R, jj = threadIdx.x / R, j = j0 + jj;
   const int row0 = a.cu[s], len = a.cu[s + 1] - row0, slot = a.slots[s];
@@ -89,60 +115,120 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
   const TQ* qg = reinterpret_cast<const TQ*>(a.q) + (long)kh * a.dk;
   const TQ* kg = reinterpret_cast<const TQ*>(a.k) + (long)kh * a.dk;
   const TQ* vg = reinterpret_cast<const TQ*>(a.v) + (long)h * a.dv;
+  auto fetch = [&](int t, TokenOps<DKT, NOPS>& x) {
+    const float* base = &ops[t][0][r * (DKT + 4)];
+#pragma unroll
+    for (int n = 0; n < NOPS; ++n)
+#pragma unroll
+      for (int c = 0; c < DKT / 4; ++c) x.v[n][c] = *reinterpret_cast<const floatx4*>(base + n * ROW + 4 * c);
+    x.vj = vs[t][jj];
+  };
+  // The next tile's operands travel from global memory into registers while this tile is computed, and
+  // into LDS once it has been consumed: the chain over the tokens never waits for a global load.
+  // (Only where a column is split over 8 or more lanes, the launch for few sequences: with the chip full,
+  // other waves cover the loads and the registers are worth more than the overlap.)
+  constexpr bool TILE_PF = R >= 8;
+  constexpr int CNT = TILE_PF ? TT * R * DKT / 256 : 1, CV = TILE_PF ? (TT * (256 / R) + 255) / 256 : 1;
+  static_assert(TT * R * DKT % 256 == 0, "a tile's operands divide evenly over the 256 threads");
+  float pf[CNT][NOPS], pv[CV];
+  auto gload = [&](int t0) {
+#pragma unroll
+    for (int c = 0; c < CNT; ++c) {
+      const int e = threadIdx.x + 256 * c, t = e / (R * DKT), i = e % (R * DKT);
+      const long row = row0 + t0 + t;
+      const bool in = i < a.dk && t0 + t < len;
+      pf[c][OQ] = in ? ldf<TQ>(qg + row * a.qs + i) : 0.f;
+      pf[c][OK] = in ? ldf<TQ>(kg + row * a.ks + i) * a.k_scale : 0.f;
+      if constexpr (FULL) {
+        pf[c][OW] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
+        pf[c][OP] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
+        pf[c][OZ] = in ? a.z[row * a.zs + (long)h * a.dk + i] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < CV; ++c) {
+      const int e = threadIdx.x + 256 * c, t = e / cols, cc = e % cols;
+      pv[c] = (t < TT && t0 + t < len && j0 + cc < a.dv) ? ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + cc) : 0.f;
+    }
+  };
+  if constexpr (TILE_PF) gload(0);
   for (int t0 = 0; t0 < len; t0 += TT) {
     const int nt = min(TT, len - t0);
     __syncthreads();  // the previous tile has been consumed
-    for (int e = threadIdx.x; e < nt * R * DKT; e += blockDim.x) {
-      const int t = e / (R * DKT), i = e % (R * DKT), li = i + 4 * (i / DKT);
-      const long row = row0 + t0 + t;
-      const bool in = i < a.dk;
-      ops[t][OQ][li] = in ? ldf<TQ>(qg + row * a.qs + i) : 0.f;
-      ops[t][OK][li] = in ? ldf<TQ>(kg + row * a.ks + i) * a.k_scale : 0.f;
-      if constexpr (FULL) {
-        ops[t][OW][li] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
-        ops[t][OP][li] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
-        ops[t][OZ][li] = in ? a.z[row * a.zs + (long)h * a.dk + i] : 0.f;
+    if constexpr (TILE_PF) {
+#pragma unroll
+      for (int c = 0; c < CNT; ++c) {
+        const int e = threadIdx.x + 256 * c, t = e / (R * DKT), i = e % (R * DKT), li = i + 4 * (i / DKT);
+#pragma unroll
+        for (int n = 0; n < NOPS; ++n) ops[t][n][li] = pf[c][n];
       }
-    }
-    for (int e = threadIdx.x; e < nt * cols; e += blockDim.x) {
-      const int t = e / cols, c = e % cols;
-      vs[t][c] = j0 + c < a.dv ? ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + c) : 0.f;
+#pragma unroll
+      for (int c = 0; c < CV; ++c) {
+        const int e = threadIdx.x + 256 * c, t = e / cols, cc = e % cols;
+        if (t < TT) vs[t][cc] = pv[c];
+      }
+    } else {
+      for (int e = threadIdx.x; e < nt * R * DKT; e += 256) {
+        const int t = e / (R * DKT), i = e % (R * DKT), li = i + 4 * (i / DKT);
+        const long row = row0 + t0 + t;
+        const bool in = i < a.dk;
+        ops[t][OQ][li] = in ? ldf<TQ>(qg + row * a.qs + i) : 0.f;
+        ops[t][OK][li] = in ? ldf<TQ>(kg + row * a.ks + i) * a.k_scale : 0.f;
+        if constexpr (FULL) {
+          ops[t][OW][li] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
+          ops[t][OP][li] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
+          ops[t][OZ][li] = in ? a.z[row * a.zs + (long)h * a.dk + i] : 0.f;
+        }
+      }
+      for (int e = threadIdx.x; e < nt * cols; e += 256) {
+        const int t = e / cols, c = e % cols;
+        vs[t][c] = j0 + c < a.dv ? ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + c) : 0.f;
+      }
     }
     __syncthreads();
-    for (int t = 0; t < nt; ++t) {
-      const float* base = &ops[t][0][r * (DKT + 4)];
-      const float vj = vs[t][jj];
+    if constexpr (TILE_PF) {
+      if (t0 + TT < len) gload(t0 + TT);
+    }
+    auto step = [&](const TokenOps<DKT, NOPS>& x, int t) {
       float zsum = 0.f;
       if constexpr (FULL) {
+        float zp[4] = {0.f, 0.f, 0.f, 0.f};   // four partial sums: four short chains of multiply-adds
 #pragma unroll
-        for (int ii = 0; ii < DKT; ii += 4) {
-          const floatx4 zz = *reinterpret_cast<const floatx4*>(base + OZ * ROW + ii);
+        for (int ii = 0; ii < DKT; ii += 4)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) zsum += zz[e] * S[ii + e];
-        }
-#pragma unroll
-        for (int o = 1; o < R; o <<= 1) zsum += __shfl_xor(zsum, o, 64);
+          for (int e = 0; e < 4; ++e) zp[e] += x.v[OZ][ii / 4][e] * S[ii + e];
+        zsum = group_sum<R>((zp[0] + zp[1]) + (zp[2] + zp[3]));
       }
-      float acc = 0.f;
+      float ap[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < DKT; ii += 4) {
-        const floatx4 kk = *reinterpret_cast<const floatx4*>(base + OK * ROW + ii);
-        const floatx4 qq = *reinterpret_cast<const floatx4*>(base + OQ * ROW + ii);
-        if constexpr (FULL) {
-          const floatx4 ww = *reinterpret_cast<const floatx4*>(base + OW * ROW + ii);
-          const floatx4 pp = *reinterpret_cast<const floatx4*>(base + OP * ROW + ii);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) S[ii + e] = ww[e] * S[ii + e] - pp[e] * zsum + kk[e] * vj;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) S[ii + e] = wh * S[ii + e] + kk[e] * vj;
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (FULL) S[ii + e] = x.v[OW][ii / 4][e] * S[ii + e] - x.v[OP][ii / 4][e] * zsum + x.v[OK][ii / 4][e] * x.vj;
+          else S[ii + e] = wh * S[ii + e] + x.v[OK][ii / 4][e] * x.vj;
+          ap[e] += x.v[OQ][ii / 4][e] * S[ii + e];
         }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc += qq[e] * S[ii + e];
       }
-#pragma unroll
-      for (int o = 1; o < R; o <<= 1) acc += __shfl_xor(acc, o, 64);
+      const float acc = group_sum<R>((ap[0] + ap[1]) + (ap[2] + ap[3]));
       if (r == 0 && live) a.o[(long)(row0 + t0 + t) * a.os + (long)h * a.dv + j] = acc;
+    };
+    if constexpr (PREFETCH) {   // two register sets in turn: the next token's operands are read under this token's arithmetic
+      TokenOps<DKT, NOPS> xa, xb;
+      fetch(0, xa);
+      for (int t = 0; t < nt; t += 2) {
+        if (t + 1 < nt) fetch(t + 1, xb);
+        step(xa, t);
+        if (t + 1 < nt) {
+          if (t + 2 < nt) fetch(t + 2, xa);
+          step(xb, t + 1);
+        }
+      }
+    } else {
+      TokenOps<DKT, NOPS> x;
+      for (int t = 0; t < nt; ++t) {
+        fetch(t, x);
+        step(x, t);
+      }
     }
   }
   if (live) {
@@ -156,10 +242,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
 
 template <typename TQ, int DKT, int R>
 int launch_scan(const ScanParams& a, int S, bool full, hipStream_t st) {
-  // columns per workgroup: up to 256 / R, no more than the state has (in whole waves)
-  const int want = ((a.dv * R + 63) / 64) * 64;
-  const int threads = want < 256 ? want : 256;
-  const int cols = threads / R;
+  constexpr int threads = 256, cols = threads / R;  // state columns per workgroup
   dim3 grid((unsigned)S, (unsigned)a.H, (unsigned)((a.dv + cols - 1) / cols));
   if (full) delta_scan_kernel<TQ, DKT, R, true><<<grid, threads, 0, st>>>(a);
   else delta_scan_kernel<TQ, DKT, R, false><<<grid, threads, 0, st>>>(a);
@@ -167,13 +250,16 @@ int launch_scan(const ScanParams& a, int S, bool full, hipStream_t st) {
   return 0;
 }
 
+// A state column is split over 4 lanes when (sequence, head) pairs alone fill the chip, over 16 when they
+// do not: the recurrence is a chain over the tokens, so with few sequences the time of a step is the work
+// of one lane per token, and more lanes per column shorten exactly that.
 template <typename TQ>
-int scan_t(const ScanParams& a, int S, bool full, hipStream_t st) {
-  if (a.dk <= 16) return launch_scan<TQ, 16, 1>(a, S, full, st);
-  if (a.dk <= 32) return launch_scan<TQ, 16, 2>(a, S, full, st);
-  if (a.dk <= 64) return launch_scan<TQ, 16, 4>(a, S, full, st);
-  if (a.dk <= 128) return launch_scan<TQ, 32, 4>(a, S, full, st);
-  if (a.dk <= 256) return launch_scan<TQ, 64, 4>(a, S, full, st);
+int scan_t(const ScanParams& a, int S, bool full, int wide, hipStream_t st) {
+  if (a.dk <= 16) return wide ? launch_scan<TQ, 4, 4>(a, S, full, st) : launch_scan<TQ, 16, 1>(a, S, full, st);
+  if (a.dk <= 32) return wide ? launch_scan<TQ, 4, 8>(a, S, full, st) : launch_scan<TQ, 16, 2>(a, S, full, st);
+  if (a.dk <= 64) return wide ? launch_scan<TQ, 4, 16>(a, S, full, st) : launch_scan<TQ, 16, 4>(a, S, full, st);
+  if (a.dk <= 128) return wide ? launch_scan<TQ, 8, 16>(a, S, full, st) : launch_scan<TQ, 32, 4>(a, S, full, st);
+  if (a.dk <= 256) return wide ? launch_scan<TQ, 16, 16>(a, S, full, st) : launch_scan<TQ, 64, 4>(a, S, full, st);
   return -1;
 }
 
@@ -292,7 +378,7 @@ __global__ __launch_bounds__(256) void tanh_kernel(T* __restrict__ x, long xs, i
 int lk_delta_scan(const void* q, long qs, const void* k, long ks, const void* v, long vs, int qkv_esz, const float* w, long ws,
                   const float* p, long ps, const float* z, long zs, const float* w_head, float k_scale, float* state,
                   const int* cu, const int* slots, const int* positions, int S, int H, int Hk, int dk, int dv, float* o, long os,
-                  hipStream_t st) {
+                  int wide, hipStream_t st) {
   if (S <= 0) return 0;
   if (H < 1 || Hk < 1 || H % Hk || dk < 1 || dk > 256 || dv < 1 || H > 65535) return -1;
   const bool full = w != nullptr;
@@ -302,7 +388,7 @@ int lk_delta_scan(const void* q, long qs, const void* k, long ks, const void* v,
   a.w = w; a.p = p; a.z = z; a.ws = ws; a.ps = ps; a.zs = zs; a.w_head = w_head; a.k_scale = k_scale;
   a.state = state; a.cu = cu; a.slots = slots; a.positions = positions; a.o = o; a.os = os;
   a.H = H; a.Hk = Hk; a.dk = dk; a.dv = dv;
-  return qkv_esz == 2 ? scan_t<bf16_t>(a, S, full, st) : scan_t<float>(a, S, full, st);
+  return qkv_esz == 2 ? scan_t<bf16_t>(a, S, full, wide, st) : scan_t<float>(a, S, full, wide, st);
 }
 
 int lk_gated_delta_prep(const void* q, long qs, const void* k, long ks, const void* v, long vs, const void* beta, long bs,

@@ -7,6 +7,8 @@
 // starts the stream, the gated tanh-GELU activation of a fused [gate | up] projection, and the mean of
 // two RMS-normed branches.  Everything is f32 arithmetic; bf16 only where a value is read from or
 // written for a GEMM.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -40,10 +42,11 @@ __global__ __launch_bounds__(256) void embed_stream_kernel(const int* __restrict
   }
 }
 
-// One workgroup per output row; thread i owns columns i, i + 256, ... (MAXI of them at most) in registers.
+// One workgroup per output row; thread i owns the column groups i, i + 256, ... of V adjacent columns (MAXI
+// groups at most) in registers; V = 4 (16-byte f32 accesses) when W % 4 == 0, else 1.
 //   idx == null: rows of x are updated in place, `out` (may be null) receives the copy in TO;
 //   idx != null: row idx[r] of x is read, nothing of x is written, out[r] receives the result.
-template <typename TY, typename TO, int MAXI>
+template <typename TY, typename TO, int MAXI, int V>
 __global__ __launch_bounds__(256) void stream_layernorm_kernel(float* __restrict__ x, const TY* __restrict__ y, long ys,
                                                                const float* __restrict__ ls, float alpha,
                                                                const float* __restrict__ w, const float* __restrict__ b,
@@ -51,37 +54,78 @@ __global__ __launch_bounds__(256) void stream_layernorm_kernel(float* __restrict
                                                                long os, int W) {
   __shared__ float red[4];
   const long orow = blockIdx.x, row = idx ? idx[orow] : orow;
-  float v[MAXI];
+  float v[MAXI][V];
   float s = 0.f;
+  auto ldn = [](const auto* p, float (&f)[V]) {   // V adjacent values as f32
+    using E = std::remove_cv_t<std::remove_reference_t<decltype(*p)>>;
+    if constexpr (V == 4 && sizeof(E) == 4) {
+      const floatx4 t = *reinterpret_cast<const floatx4*>(p);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f[e] = t[e];
+    } else if constexpr (V == 4) {
+      const short4_t t = *reinterpret_cast<const short4_t*>(p);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f[e] = bf2f((bf16_t)t[e]);
+    } else {
+      f[0] = ldv<E>(p);
+    }
+  };
 #pragma unroll
   for (int i = 0; i < MAXI; ++i) {
-    const int c = threadIdx.x + 256 * i;
-    v[i] = 0.f;
+    const int c = (threadIdx.x + 256 * i) * V;
+#pragma unroll
+    for (int e = 0; e < V; ++e) v[i][e] = 0.f;
     if (c < W) {
-      float t = x[row * W + c];
-      if (y) t = alpha * t + (ls ? ls[c] : 1.f) * ldv<TY>(y + row * ys + c);
-      v[i] = t;
-      s += t;
+      ldn(x + row * W + c, v[i]);
+      if (y) {
+        float yy[V], ll[V];
+        ldn(y + row * ys + c, yy);
+        if (ls) ldn(ls + c, ll);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[i][e] = alpha * v[i][e] + (ls ? ll[e] : 1.f) * yy[e];
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) s += v[i][e];
     }
   }
   const float mean = block_sum<4>(s, red) / (float)W;
   float q = 0.f;
 #pragma unroll
   for (int i = 0; i < MAXI; ++i) {
-    const int c = threadIdx.x + 256 * i;
-    if (c < W) {
-      v[i] -= mean;
-      q += v[i] * v[i];
+    if ((threadIdx.x + 256 * i) * V < W) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        v[i][e] -= mean;
+        q += v[i][e] * v[i][e];
+      }
     }
   }
   const float inv = 1.f / sqrtf(block_sum<4>(q, red) / (float)W + eps);
 #pragma unroll
   for (int i = 0; i < MAXI; ++i) {
-    const int c = threadIdx.x + 256 * i;
+    const int c = (threadIdx.x + 256 * i) * V;
     if (c < W) {
-      const float r = v[i] * inv * w[c] + b[c];
-      if (!idx) x[row * W + c] = r;
-      if (out) stv<TO>(out + orow * os + c, r);
+      float ww[V], bb[V], r[V];
+      ldn(w + c, ww);
+      ldn(b + c, bb);
+#pragma unroll
+      for (int e = 0; e < V; ++e) r[e] = v[i][e] * inv * ww[e] + bb[e];
+      if constexpr (V == 4) {
+        if (!idx) *reinterpret_cast<floatx4*>(x + row * W + c) = floatx4{r[0], r[1], r[2], r[3]};
+        if (out) {
+          if constexpr (sizeof(TO) == 4) {
+            *reinterpret_cast<floatx4*>(out + orow * os + c) = floatx4{r[0], r[1], r[2], r[3]};
+          } else {
+            short4_t t;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[e] = (short)f2bf(r[e]);
+            *reinterpret_cast<short4_t*>(out + orow * os + c) = t;
+          }
+        }
+      } else {
+        if (!idx) x[row * W + c] = r[0];
+        if (out) stv<TO>(out + orow * os + c, r[0]);
+      }
     }
   }
 }
@@ -122,13 +166,23 @@ __global__ __launch_bounds__(256) void dual_rmsnorm_mean_kernel(const T* __restr
 template <typename TY, typename TO>
 int launch_ln(float* x, const void* y, long ys, const float* ls, float alpha, const float* w, const float* b, float eps,
               const long* idx, void* out, long os, long rows, int W, hipStream_t st) {
-#define LK_LN(MAXI)                                                                                                            \
-  stream_layernorm_kernel<TY, TO, MAXI><<<(unsigned)rows, 256, 0, st>>>(x, (const TY*)y, ys, ls, alpha, w, b, eps, idx, (TO*)out, \
-                                                                        os, W)
-  if (W <= 1024) LK_LN(4);
-  else if (W <= 4096) LK_LN(16);
-  else if (W <= 16384) LK_LN(64);
-  else return -1;
+  // 16-byte accesses need whole groups of 4 columns and rows that start on 16-byte (f32) / 8-byte (bf16) borders
+  const bool vec = W % 4 == 0 && (!y || (ys % 4 == 0 && (uintptr_t)y % 16 == 0)) && (!out || (os % 4 == 0 && (uintptr_t)out % 16 == 0)) &&
+                   (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)b % 16 == 0 && (!ls || (uintptr_t)ls % 16 == 0);
+#define LK_LN(MAXI, V)                                                                                                            \
+  stream_layernorm_kernel<TY, TO, MAXI, V><<<(unsigned)rows, 256, 0, st>>>(x, (const TY*)y, ys, ls, alpha, w, b, eps, idx, (TO*)out, \
+                                                                           os, W)
+  if (vec) {
+    if (W <= 1024) LK_LN(1, 4);
+    else if (W <= 4096) LK_LN(4, 4);
+    else if (W <= 16384) LK_LN(16, 4);
+    else return -1;
+  } else {
+    if (W <= 1024) LK_LN(4, 1);
+    else if (W <= 4096) LK_LN(16, 1);
+    else if (W <= 16384) LK_LN(64, 1);
+    else return -1;
+  }
 #undef LK_LN
   LK_CHECK_LAUNCH();
   return 0;
