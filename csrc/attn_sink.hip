@@ -73,21 +73,45 @@ LK_DEVICE void sink_run(const SinkParams& p, const uint4_t (&qf)[PAD / (4 * El<T
   const T* kc = reinterpret_cast<const T*>(p.kc);
   const T* vc = reinterpret_cast<const T*>(p.vc);
   const int krow = 8 * (n16 >> 2) + (n16 & 3);
-  for (int kb = k0 + 32 * step0; kb < k1; kb += 32 * stride) {
-    floatx4 c[2];
+  // bf16: the next step's K fragments are requested as soon as this step's Q.K products have consumed the
+  // current ones, and this step's V fragments before the softmax arithmetic, so both fly under it
+  auto load_k = [&](int kb, uint4_t (&kf)[2][KS]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int key = min(kb + krow + 4 * t, k1 - 1);
       const T* kr = kc + (((long)bt[key / p.BS] * p.G + kvh) * p.BS + key % p.BS) * p.dim;
-      c[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const int d0 = s * 4 * EV + g * EV;
-        if (s * 4 * EV < p.dim) c[t] = mma_qk<T>(d0 < p.dim ? ld16(kr + d0) : uint4_t{0u, 0u, 0u, 0u}, qf[s], c[t]);
+        kf[t][s] = d0 < p.dim ? ld16(kr + d0) : uint4_t{0u, 0u, 0u, 0u};
       }
+    }
+  };
+  uint4_t kf[2][KS];
+  int kb = k0 + 32 * step0;
+  if (BF && kb < k1) load_k(kb, kf);
+  for (; kb < k1; kb += 32 * stride) {
+    if (!BF) load_k(kb, kf);
+    floatx4 c[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      c[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        if (s * 4 * EV < p.dim) c[t] = mma_qk<T>(kf[t][s], qf[s], c[t]);
     }
     const int vk = kb + 8 * g < k1 ? kb + 8 * g : ((k1 - 1) & ~7);
     const T* vrow = vc + ((long)bt[vk / p.BS] * p.G + kvh) * p.vdim * p.BS + vk % p.BS;
+    uint4_t vf[BF ? VT : 1];
+    if constexpr (BF) {
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        const int vd = vt * 16 + n16;
+        vf[vt] = (vt * 16 < p.vdim && vd < p.vdim) ? ld16(vrow + (long)vd * p.BS) : uint4_t{0u, 0u, 0u, 0u};
+      }
+      const int kn = kb + 32 * stride;
+      if (kn < k1) load_k(kn, kf);
+    }
     float sc[2][4];
     bool ok[2][4];
     float mx = kNegBig;
@@ -127,11 +151,7 @@ LK_DEVICE void sink_run(const SinkParams& p, const uint4_t (&qf)[PAD / (4 * El<T
       }
 #pragma unroll
       for (int vt = 0; vt < VT; ++vt)
-        if (vt * 16 < p.vdim) {
-          const int vd = vt * 16 + n16;
-          const uint4_t vf = vd < p.vdim ? ld16(vrow + (long)vd * p.BS) : uint4_t{0u, 0u, 0u, 0u};
-          o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(short8, vf), pbits, o[vt], 0, 0, 0);
-        }
+        if (vt * 16 < p.vdim) o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(short8, vf[vt]), pbits, o[vt], 0, 0, 0);
     } else {
 #pragma unroll
       for (int vt = 0; vt < VT; ++vt) {
