@@ -1346,7 +1346,7 @@ const float* f32_rows(const c10::optional<at::Tensor>& t, long T, long n, const 
 at::Tensor delta_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& w,
                       const c10::optional<at::Tensor>& p, const c10::optional<at::Tensor>& z, at::Tensor& state, const at::Tensor& cu,
                       const at::Tensor& slots, const at::Tensor& positions, int64_t H, int64_t Hk, int64_t dk, int64_t dv,
-                      const c10::optional<at::Tensor>& w_head, double k_scale, int64_t max_len) {
+                      const c10::optional<at::Tensor>& w_head, double k_scale, int64_t max_len, int64_t lanes) {
   const long T = q.size(0);
   TORCH_CHECK(H >= 1 && Hk >= 1 && H % Hk == 0 && dk >= 1 && dk <= 256 && dv >= 1, "delta_scan sizes");
   check_rows(q, T, Hk * dk, "q"); check_rows(k, T, Hk * dk, "k"); check_rows(v, T, H * dv, "v");
@@ -1364,7 +1364,8 @@ at::Tensor delta_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
   at::Tensor o = at::empty({T, H * dv}, q.options().dtype(at::kFloat));
   // few (sequence, head) pairs: 16 lanes per state column instead of 4 (a static function of the step's shape)
   const long S = cu.numel() - 1;
-  const int wide = S * H * ((dv * 4 + 255) / 256) < 2 * 256 ? 1 : 0;
+  // (lanes: 4 or 16 forces one of the two forms -- tests; anything else: by the step's shape)
+  const int wide = lanes == 16 ? 1 : lanes == 4 ? 0 : (S * H * ((dv * 4 + 255) / 256) < 2 * 256 ? 1 : 0);
   CHECK_RC(lk_delta_scan(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), esz, wp, ws, pp, ps, zp, zs,
                          wp ? nullptr : fpo(w_head, H, "w_head"), (float)k_scale, state.data_ptr<float>(), ip(cu), ip(slots),
                          ip(positions), cu.numel() - 1, (int)H, (int)Hk, (int)dk, (int)dv, o.data_ptr<float>(), o.stride(0),

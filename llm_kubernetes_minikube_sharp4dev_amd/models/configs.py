@@ -192,7 +192,7 @@ def pemidra_layers(n: int, heads: int, head_dim: int, ff: int, kv_heads: Optiona
         t = pattern[i % len(pattern)]
         if t == "retention":
             mixer = {"heads": heads, "dim": head_dim, "vdim": head_dim,
-                     "decay": [1.0 - 2.0 ** (-5 - (j % 8)) for j in range(heads)]}
+                     "decay": [0.9 + 0.0125 * (j % 8) for j in range(heads)]}
         elif t == "general_delta":
             mixer = {"heads": heads, "dim": head_dim, "lora": lora}
         else:

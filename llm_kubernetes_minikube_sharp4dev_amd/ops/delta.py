@@ -37,14 +37,16 @@ def delta_scan_supported(dk: int, dv: int) -> bool:
 
 
 def delta_scan(q, k, v, w, p, z, state, cu, slots, positions, H: int, Hk: int, dk: int, dv: int,
-               w_head=None, k_scale: float = 1.0, max_len: int = 1):
+               w_head=None, k_scale: float = 1.0, max_len: int = 1, lanes: int = 0):
     """o f32 [T, H * dv] of the recurrence in the module docstring, per sequence and head, the state read
     from / left in ``state[slot]``.  q, k: rows of ``Hk * dk`` (head h reads q/k head ``h // (H / Hk)``),
     v: rows of ``H * dv``; each in bf16 or f32 (k is multiplied by ``k_scale`` in f32).  ``w``: f32 rows of
     ``H * dk``, or None with ``w_head`` f32 [H] (one decay per head).  ``p``, ``z``: f32 rows of ``H * dk``,
-    or both None (no removal term)."""
+    or both None (no removal term).  ``lanes``: 4 or 16 forces how many lanes of the GPU kernel share a state
+    column (default: by the step's shape -- 16 while (sequence, head) pairs do not fill the chip)."""
     if use_hip(q):
-        return lib().delta_scan(q, k, v, w, p, z, state, cu, slots, positions, H, Hk, dk, dv, w_head, float(k_scale), int(max_len))
+        return lib().delta_scan(q, k, v, w, p, z, state, cu, slots, positions, H, Hk, dk, dv, w_head, float(k_scale), int(max_len),
+                                int(lanes))
     T = q.shape[0]
     o = torch.zeros(T, H * dv, dtype=torch.float32, device=q.device)
     cul, sl = cu.tolist(), slots.tolist()

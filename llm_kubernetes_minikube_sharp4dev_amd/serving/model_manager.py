@@ -24,7 +24,7 @@ import torch
 from ..config import Config
 from ..engine.embed_engine import EmbeddingEngine
 from ..engine.llm_engine import AsyncLLMEngine, LLMEngine
-from ..models import build_decoder, build_encoder, checkpoint_architecture, load_decoder_dir
+from ..models import NATIVE_CONFIGS, build_decoder, build_encoder, checkpoint_architecture, load_decoder_dir
 from ..models.configs import DECODERS, ENCODERS, param_count
 from ..models.tokenizer import load_tokenizer
 from ..utils.logging import get_logger
@@ -142,8 +142,8 @@ class ModelManager:
 
     def _build_generator(self, name: str, preset: str):
         ck = self.checkpoints.get(name) or self.checkpoints.get(preset)
-        if ck and checkpoint_architecture(ck) == "lebepel":
-            # a hybrid checkpoint brings its own config.json (sizes, layer order, constants): the preset only named it
+        if ck and checkpoint_architecture(ck) in NATIVE_CONFIGS:
+            # such a checkpoint brings its own config.json (sizes, layer order, constants): the preset only named it
             return load_decoder_dir(ck, device=self.device, dtype=self._dtype()), load_tokenizer(ck)
         model = build_decoder(preset, device=self.device, seed=self.cfg.engine.seed, checkpoint=ck, dtype=self._dtype(),
                               **({"tp": self.tp} if self.tp is not None else {}))

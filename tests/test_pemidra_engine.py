@@ -306,10 +306,13 @@ def test_captured_decode_graph_matches_the_oracle():
         assert ok, err
 
 
-def test_served_through_the_model_manager():
+def test_served_through_the_model_manager(tmp_path):
     """The serving stack's model manager builds the preset, wraps it in an engine with state slots and
-    prefix caching off, and generates through the server's pipelined step loop."""
+    prefix caching off, and generates through the server's pipelined step loop; a checkpoint directory
+    given for a served name brings its own config."""
     import asyncio
+
+    from safetensors.torch import save_file
 
     from llm_kubernetes_minikube_sharp4dev_amd.config import Config
     from llm_kubernetes_minikube_sharp4dev_amd.serving.model_manager import ModelManager
@@ -336,3 +339,14 @@ def test_served_through_the_model_manager():
         full = prompt + list(sq.output_ids)
         lg = O.forward(eng.model.cfg.to_json(), sd, full[:-1])[len(prompt) - 1:]
         assert [int(x) for x in lg.argmax(-1)] == list(sq.output_ids)
+    _, sd_odd = model_and_weights("odd", "cpu", torch.float32)
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(CONFIGS["odd"]))
+    save_file({k: v.to(torch.bfloat16) for k, v in sd_odd.items()}, str(d / "model.safetensors"))
+    mgr2 = ModelManager(cfg, device="cpu", checkpoints={"pemidra-tiny": str(d)}, engine_overrides={"num_blocks": 32})
+    h2 = mgr2.generator("pemidra-tiny")
+    try:
+        assert isinstance(h2.engine.model, PemidraModel) and h2.engine.model.cfg.hidden == 36 and h2.engine.model.cfg.vocab_size == 61
+    finally:
+        h2.async_engine.shutdown()

@@ -177,6 +177,52 @@ def test_state_slots_start_from_zero_and_are_independent(device, dtype):
         assert rel_err(got, fn(hh, sd, "l0.mix.", mixer, 1e-5)) < tol(dtype)
 
 
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("dk,dv,H,Hk", [(8, 10, 2, 1), (24, 16, 4, 2), (48, 64, 2, 2), (96, 40, 3, 1), (200, 72, 1, 1)])
+def test_scan_forms_agree_with_the_recurrence(dk, dv, H, Hk, device, dtype):
+    """The scan op alone, both lane splits of the GPU kernel (4 and 16 lanes per state column), with and
+    without the removal term, two sequences of unequal length continued from an earlier state, against the
+    recurrence written out in float64."""
+    g = torch.Generator().manual_seed(dk)
+    lens, T = [19, 6], 25
+    q, k, v = q16(rnd(g, T, Hk * dk, scale=0.4)), q16(rnd(g, T, Hk * dk, scale=0.4)), q16(rnd(g, T, H * dv))
+    w = torch.rand(T, H * dk, generator=g, dtype=torch.float64).float().double() * 0.5 + 0.5
+    p, z = rnd(g, T, H * dk, scale=0.3).float().double(), rnd(g, T, H * dk, scale=0.3).float().double()
+    wh = torch.tensor([0.9, 1.0, 0.5, 0.75][:H], dtype=torch.float64)
+    S0 = rnd(g, 3, H, dk, dv, scale=0.2).float().double()
+    i32 = dict(dtype=torch.int32, device=device)
+    cu, slots = torch.tensor([0, 19, 25], **i32), torch.tensor([2, 0], **i32)
+    pos = torch.tensor(list(range(5, 24)) + list(range(0, 6)), **i32)      # the first continues, the second starts fresh
+    for full in (True, False):
+        want = torch.zeros(T, H, dv, dtype=torch.float64)
+        end = {}
+        for s, (r0, n, slot, fresh) in enumerate(((0, 19, 2, False), (19, 6, 0, True))):
+            for h in range(H):
+                S = torch.zeros(dk, dv, dtype=torch.float64) if fresh else S0[slot, h].clone()
+                kh = h // (H // Hk)
+                for t in range(r0, r0 + n):
+                    kk = k[t, kh * dk:(kh + 1) * dk] * (1.0 if full else 0.5)
+                    if full:
+                        S = w[t, h * dk:(h + 1) * dk, None] * S - torch.outer(p[t, h * dk:(h + 1) * dk], S.T @ z[t, h * dk:(h + 1) * dk]) \
+                            + torch.outer(kk, v[t, h * dv:(h + 1) * dv])
+                    else:
+                        S = wh[h] * S + torch.outer(kk, v[t, h * dv:(h + 1) * dv])
+                    want[t, h] = S.T @ q[t, kh * dk:(kh + 1) * dk]
+                end[(slot, h)] = S
+        for lanes in ((0,) if device == "cpu" else (0, 4, 16)):
+            for qdt in (dtype, torch.float32):          # operands in the activation dtype, and as the f32 the operand kernels write
+                state = S0.float().to(device).clone()
+                f = lambda t: t.float().to(device)      # noqa: E731
+                c = lambda t: t.to(qdt).to(device)      # noqa: E731
+                got = ops.delta_scan(c(q), c(k), c(v), f(w) if full else None, f(p) if full else None, f(z) if full else None, state, cu,
+                                     slots, pos, H, Hk, dk, dv, w_head=None if full else f(wh), k_scale=1.0 if full else 0.5, max_len=19,
+                                     lanes=lanes)
+                assert rel_err(got.view(T, H, dv), want) < 2e-5, (full, lanes, qdt)
+                for (slot, h), S in end.items():
+                    assert rel_err(state[slot, h], S) < 2e-5
+                assert torch.equal(state[1].cpu(), S0[1].float())      # a slot no sequence holds is not touched
+
+
 # ---------------------------------------------------------------------------- attention: mask edges, sink, far keys
 def attend(q, k, v, qpos, hscale, first, sink=True):
     """Plain softmax with one more term of score 0 in the denominator: q [H, d] at position qpos over
