@@ -42,9 +42,10 @@ class FusedRows:
 
 
 def fused_mult(width: int) -> int:
-    """Row multiple of a fused projection: the decode-sized GEMM kernels tile 128 output columns and need
-    a contraction size that is a multiple of 256; other widths run on kernels without that constraint."""
-    return 128 if width % 256 == 0 else 8
+    """Row multiple of a fused projection: the framework's GEMM kernels tile 256 output columns for prompt
+    portions and 128 for decode-sized steps, and the latter need a contraction size that is a multiple of
+    256; other widths run on kernels without that constraint."""
+    return 256 if width % 256 == 0 else 8
 
 
 @dataclass
