@@ -1,6 +1,8 @@
 """Entry points of the sequence-mixer kernels beside softmax attention: an f32 residual stream
 (``csrc/stream_f32.hip``), sigmoid attention with a log-distance penalty over a paged cache
-(``csrc/attn_sigmoid.hip``) and a Mamba-2 style state-space mixer (``csrc/ssm.hip``).
+(``csrc/attn_sigmoid.hip``), a Mamba-2 style state-space mixer (``csrc/ssm.hip``), a post-norm f32
+stream with layer norms (``csrc/stream_ln.hip``) and softmax attention with a sink under a causal / chunk /
+window mask over the same paged cache (``csrc/attn_sink.hip``).  The linear-state scans are in ``ops.delta``.
 
 GPU tensors go to the HIP kernels (bf16 or f32 activations); CPU tensors to the torch
 implementations below, which keep the kernels' layouts and their split of what is 32-bit:
